@@ -1,0 +1,229 @@
+/*
+ * tnn_hip.h -- C ABI of the MI355X (gfx950) implementation of tiny-dpcpp-nn's hot path:
+ * the fully fused MLP (inference / training forward / fused backward with weight gradients),
+ * the L2 loss, an Adam step, and the multi-resolution hash-grid encoding (forward / backward).
+ *
+ * Conventions
+ *  - Every pointer named d_* is DEVICE memory owned by the caller. The library keeps no state,
+ *    allocates nothing and is thread-safe; every call is asynchronous on `stream`
+ *    (a hipStream_t passed as void*, NULL = the default stream).
+ *  - Return value: 0 on success, a negative tnn_status otherwise. No exception crosses this
+ *    boundary; tnn_last_error() returns a thread-local message for the last failure.
+ *  - "T" is the 2-byte storage type selected by tnn_mlp_desc::dtype (bf16 or fp16); all
+ *    contractions accumulate in fp32 (reference: include/network/kernel_esimd.h:92-105).
+ *  - Activation codes are the ordinals of the reference's `enum class Activation`
+ *    (include/common/common.h:28-38); only None, ReLU and Sigmoid are accepted, as in
+ *    include/network/SwiftNetMLP.h:252-291.
+ *
+ * Each entry point cites the reference interface it stands in for (paths relative to the
+ * reference checkout).
+ */
+#ifndef TNN_HIP_H
+#define TNN_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TNN_HIP_ABI_VERSION 1
+
+typedef void *tnn_stream_t; /* hipStream_t */
+
+typedef enum tnn_status {
+    TNN_OK = 0,
+    TNN_ERR_INVALID_ARGUMENT = -1, /* reference: std::invalid_argument / std::runtime_error in the checks cited below */
+    TNN_ERR_UNSUPPORTED = -2,      /* a variant the reference does not instantiate either */
+    TNN_ERR_HIP = -3,              /* a HIP runtime call failed (launch error, no device, wrong architecture) */
+    TNN_ERR_WORKSPACE = -4         /* workspace missing or too small */
+} tnn_status;
+
+typedef enum tnn_dtype { TNN_BF16 = 0, TNN_FP16 = 1, TNN_FP32 = 2 } tnn_dtype;
+
+/* include/common/common.h:28-38 */
+typedef enum tnn_activation {
+    TNN_ACT_RELU = 0,
+    TNN_ACT_LEAKY_RELU = 1,
+    TNN_ACT_EXPONENTIAL = 2,
+    TNN_ACT_SINE = 3,
+    TNN_ACT_SIGMOID = 4,
+    TNN_ACT_SQUAREPLUS = 5,
+    TNN_ACT_SOFTPLUS = 6,
+    TNN_ACT_TANH = 7,
+    TNN_ACT_NONE = 8
+} tnn_activation;
+
+/* Shape of one fused MLP. Stands in for the template/ctor arguments of
+ * SwiftNetMLP<T, WIDTH>(q, in, out, n_hidden_layers, activation, output_activation)
+ * (include/network/SwiftNetMLP.h:50-67) after padding input and output to `width`
+ * (include/network/Network.h:64-82). The network has n_hidden_layers + 1 weight matrices,
+ * each width x width. width in {16, 32, 64, 128} (include/network/Network.h:160-161). */
+typedef struct tnn_mlp_desc {
+    int32_t dtype;             /* TNN_BF16 or TNN_FP16 */
+    int32_t width;             /* 16, 32, 64, 128 */
+    int32_t n_hidden_layers;   /* >= 1 */
+    int32_t activation;        /* hidden layers */
+    int32_t output_activation; /* last layer */
+} tnn_mlp_desc;
+
+const char *tnn_last_error(void);
+int tnn_abi_version(void);
+/* Number of HIP devices whose architecture is gfx950, or a negative status. */
+int tnn_device_check(void);
+
+/* ------------------------------------------------------------------------------------------
+ * Weight layouts.
+ *   unpacked : per matrix element (k=in, n=out) at k*W + n (test/mlp.h:391-402)
+ *   packed   : per matrix element (k, n) at (k & ~1)*W + 2n + (k & 1); the layout of the reference's
+ *              parameters, get_params() and gradients (source/common/common.cpp:33-66)
+ *   prepared : the MFMA operand order the kernels read; opaque, produced only by
+ *              tnn_mlp_prepare_weights. It plays the role of the reference's second device copy,
+ *              m_weightsT_matrices (include/network/Network.h:76-77,235-238).
+ * ------------------------------------------------------------------------------------------ */
+
+/* get_packed_weights (include/common/common.h:184-212), on device, n_mats W x W matrices of T. */
+int tnn_pack_weights(int dtype, int width, int n_mats, const void *d_unpacked, void *d_packed, tnn_stream_t stream);
+/* inverse of the above (fromPackedLayoutCoord, source/common/common.cpp:58-66). */
+int tnn_unpack_weights(int dtype, int width, int n_mats, const void *d_packed, void *d_unpacked, tnn_stream_t stream);
+/* DeviceMatrices::PackedTranspose (include/common/DeviceMatrix.h:429-444): packed W -> packed W^T. */
+int tnn_packed_transpose(int dtype, int width, int n_mats, const void *d_packed, void *d_packed_T, tnn_stream_t stream);
+/* DeviceMatrices::PackAndTranspose (include/common/DeviceMatrix.h:469-488): raw gradients
+ * [out][in] -> parameter layout. In-place (d_raw == d_packed) is NOT allowed. */
+int tnn_pack_and_transpose(int dtype, int width, int n_mats, const void *d_raw, void *d_packed, tnn_stream_t stream);
+/* Network::ZeroWeightsPadding (include/network/Network.h:171-233) on packed weights: zero the rows of
+ * matrix 0 at and beyond the one-padded input width, and the columns of the last matrix at and
+ * beyond the unpadded output width. */
+int tnn_zero_weights_padding(const tnn_mlp_desc *desc, void *d_packed, int unpadded_input_width,
+                             int unpadded_output_width, int use_bias, tnn_stream_t stream);
+
+/* Bytes of ONE prepared buffer (forward and backward operand sets have the same size). */
+size_t tnn_mlp_prepared_bytes(const tnn_mlp_desc *desc);
+/* Packed parameters (type T, or fp32 master weights when src_is_fp32 != 0; they are rounded to T) ->
+ * prepared forward and backward operand sets. Either output may be NULL. Replaces the device-side
+ * work of Network::set_weights_matrices + TransposeWeights (include/network/Network.h:90-112). */
+int tnn_mlp_prepare_weights(const tnn_mlp_desc *desc, const void *d_packed, int src_is_fp32, void *d_prepared_fwd,
+                            void *d_prepared_bwd, tnn_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Fused MLP. Batch size M must be a multiple of 8 (include/network/SwiftNetMLP.h:293-300).
+ * ------------------------------------------------------------------------------------------ */
+
+/* EsimdKernels::inference_impl (include/network/kernel_esimd.h:242-247,565-640) reached through
+ * SwiftNetMLP::inference (include/network/SwiftNetMLP.h:135-179).
+ *   d_x: M x W row-major T. d_y: M x W row-major T (matrix 0 of the reference's output view). */
+int tnn_mlp_inference(const tnn_mlp_desc *desc, const void *d_prepared_fwd, const void *d_x, void *d_y, size_t M,
+                      tnn_stream_t stream);
+
+/* EsimdKernels::forward_impl (include/network/kernel_esimd.h:153-158,565-640) reached through
+ * SwiftNetMLP::forward_pass (include/network/SwiftNetMLP.h:69-119).
+ *   d_interm_fwd: (n_hidden_layers + 2) matrices M x W: [0] = copy of x, [l] = activated output of
+ *   matrix l-1, last = network output (include/common/DeviceMatrix.h:76-94). */
+int tnn_mlp_forward(const tnn_mlp_desc *desc, const void *d_prepared_fwd, const void *d_x, void *d_interm_fwd, size_t M,
+                    tnn_stream_t stream);
+
+/* Workspace bytes tnn_mlp_backward / tnn_mlp_train_step_l2 need for their per-workgroup fp32
+ * partial weight gradients. */
+size_t tnn_mlp_backward_workspace_bytes(const tnn_mlp_desc *desc, size_t M);
+
+/* EsimdKernels::backward_impl (include/network/kernel_esimd.h:160-240: fused delta propagation
+ * followed by oneMKL gemm_batch for dW) reached through SwiftNetMLP::backward_pass
+ * (include/network/SwiftNetMLP.h:199-248).
+ *   d_dLdy: M x W T. d_interm_fwd: as written by tnn_mlp_forward.
+ *   d_interm_bwd: (n_hidden_layers + 1) matrices M x W, [l] = delta_l; may be NULL (then the deltas
+ *                 never leave the chip).
+ *   d_dW: (n_hidden_layers + 1) matrices [n=out][k=in] row-major T, unpacked (the gemm_batch output).
+ *         If dW_is_fp32 != 0 the same layout is written as fp32 without the final rounding.
+ *   d_dLdx: M x W T or NULL (kernel_esimd.h:217-226). */
+int tnn_mlp_backward(const tnn_mlp_desc *desc, const void *d_prepared_bwd, const void *d_dLdy,
+                     const void *d_interm_fwd, void *d_interm_bwd, void *d_dW, int dW_is_fp32, void *d_dLdx, size_t M,
+                     void *d_workspace, size_t workspace_bytes, tnn_stream_t stream);
+
+/* L2Loss (include/losses/l2.h:19-40, include/losses/loss.h:19-25): value_i = (p_i - t_i)^2 / N,
+ * grad_i = T(loss_scale * 2 (p_i - t_i) / N), N = n_elements. d_values (fp32) may be NULL. */
+int tnn_l2_loss(int dtype, const void *d_predictions, const float *d_targets, size_t n_elements, float loss_scale,
+                float *d_values, void *d_grads, tnn_stream_t stream);
+
+/* One fused training step of the MLP: forward, L2 loss against fp32 targets, backward with weight
+ * gradients, with no activation or delta written to device memory. Equivalent to
+ * Trainer::training_step (include/trainer.h:23-46) with L2Loss::evaluate in between.
+ *   d_y: M x W network output (T) or NULL. d_loss_sum: one fp32 that receives sum_i value_i
+ *   (the mean squared error), or NULL. d_dW / dW_is_fp32 / d_dLdx as in tnn_mlp_backward.
+ *   N of the loss = M * W (all padded columns count, as in the reference). */
+int tnn_mlp_train_step_l2(const tnn_mlp_desc *desc, const void *d_prepared_fwd, const void *d_prepared_bwd,
+                          const void *d_x, const float *d_targets, float loss_scale, void *d_y, float *d_loss_sum,
+                          void *d_dW, int dW_is_fp32, void *d_dLdx, size_t M, void *d_workspace,
+                          size_t workspace_bytes, tnn_stream_t stream);
+
+/* Adam on fp32 master parameters with the semantics of torch.optim.Adam (the optimizer the reference's
+ * training loops use: dpcpp_bindings/tiny_dpcpp_nn/modules.py:171-175,
+ * test/python/test_compare_torch_dpcpp.py:37). grad_dtype selects how d_grad is read (T or fp32);
+ * grad is multiplied by grad_scale first (1/loss_scale). step counts from 1. If d_param_T is not NULL
+ * it receives the updated parameters rounded to param_T_dtype. */
+int tnn_adam_step(float *d_param, float *d_m, float *d_v, const void *d_grad, int grad_dtype, float grad_scale,
+                  size_t n, int step, float lr, float beta1, float beta2, float eps, void *d_param_T,
+                  int param_T_dtype, tnn_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Multi-resolution hash grid (include/encodings/grid.h, include/common/common_device.h:700-775).
+ * ------------------------------------------------------------------------------------------ */
+#define TNN_GRID_MAX_LEVELS 128 /* include/encodings/grid_interface.h:23 */
+
+typedef enum tnn_grid_type { TNN_GRID_HASH = 0, TNN_GRID_DENSE = 1, TNN_GRID_TILED = 2 } tnn_grid_type;
+typedef enum tnn_hash_type {
+    TNN_HASH_PRIME = 0,
+    TNN_HASH_COHERENT_PRIME = 1,
+    TNN_HASH_REVERSED_PRIME = 2,
+    TNN_HASH_RNG = 3
+} tnn_hash_type;
+typedef enum tnn_interpolation { TNN_INTERP_NEAREST = 0, TNN_INTERP_LINEAR = 1, TNN_INTERP_SMOOTHSTEP = 2 } tnn_interpolation;
+
+/* Everything kernel_grid / kernel_grid_backward receive by value (include/encodings/grid.h:37-47,
+ * GridOffsetTable include/encodings/grid_interface.h:24-28). Filled by tnn_grid_desc_init, which does
+ * the work of the GridEncodingTemplated constructor (include/encodings/grid.h:588-659) on the host:
+ * the per-level scale and resolution are evaluated once with the host's float math. */
+typedef struct tnn_grid_desc {
+    uint32_t n_dims;               /* 2 or 3 */
+    uint32_t n_levels;             /* <= TNN_GRID_MAX_LEVELS */
+    uint32_t n_features_per_level; /* 1, 2, 4 or 8 */
+    uint32_t log2_hashmap_size;
+    uint32_t base_resolution;
+    float per_level_scale;
+    uint32_t grid_type;
+    uint32_t hash_type;
+    uint32_t interpolation;
+    uint32_t param_dtype; /* dtype of the table: TNN_FP32 (reference) or TNN_FP16 */
+    uint32_t offsets[TNN_GRID_MAX_LEVELS + 1]; /* in entries; entry e of level l holds its features at (offsets[l]+e)*F */
+    float scales[TNN_GRID_MAX_LEVELS];
+    uint32_t resolutions[TNN_GRID_MAX_LEVELS];
+} tnn_grid_desc;
+
+int tnn_grid_desc_init(tnn_grid_desc *desc, uint32_t n_dims, uint32_t n_levels, uint32_t n_features_per_level,
+                       uint32_t log2_hashmap_size, uint32_t base_resolution, float per_level_scale,
+                       uint32_t grid_type, uint32_t hash_type, uint32_t interpolation, uint32_t param_dtype);
+/* offsets[n_levels] * n_features_per_level */
+size_t tnn_grid_n_params(const tnn_grid_desc *desc);
+
+/* kernel_grid + the zero padding kernel (include/encodings/grid.h:37-135,661-734).
+ *   d_x: M x n_dims fp32 row-major. d_table: n_params of param_dtype.
+ *   d_out: M x padded_width of out_dtype (TNN_FP32 as in the reference, or TNN_BF16/TNN_FP16 so the
+ *   MLP can consume it without a cast); column l*F + f, columns >= n_levels*F zero. */
+int tnn_grid_forward(const tnn_grid_desc *desc, const float *d_x, const void *d_table, void *d_out, int out_dtype,
+                     uint32_t padded_width, size_t M, tnn_stream_t stream);
+
+/* kernel_grid_backward with GradientMode::Overwrite or Accumulate (include/encodings/grid.h:137-245,
+ * 736-797). d_dLdy: M x padded_width of dy_dtype. d_grad_table: n_params fp32 (grad_t = float,
+ * grid.h:586). overwrite != 0 zeroes the table first (grid.h:758-762). */
+int tnn_grid_backward(const tnn_grid_desc *desc, const float *d_x, const void *d_dLdy, int dy_dtype,
+                      uint32_t padded_width, float *d_grad_table, int overwrite, size_t M, tnn_stream_t stream);
+
+/* Debug/verification aid: entry index (inside its level) of every (point, level, corner), the
+ * integer part of kernel_grid (grid.h:95-129 with grid_index, common_device.h:745-765).
+ * d_indices: M x n_levels x 2^n_dims uint32. */
+int tnn_grid_indices(const tnn_grid_desc *desc, const float *d_x, uint32_t *d_indices, size_t M, tnn_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TNN_HIP_H */

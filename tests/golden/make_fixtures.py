@@ -1,0 +1,69 @@
+"""Writes the golden fixtures under tests/golden/ from the data the reference's own tests hold.
+
+Run in the build container (needs /root/reference as TEXT only; nothing of the reference is imported
+or executed). The fixtures are data: expected output vectors and the parameters that produce them.
+"""
+import json
+import os
+import re
+
+REF = "/root/reference"
+HERE = os.path.dirname(os.path.abspath(__file__))
+
+
+def numbers_between(text, start_marker, end_marker):
+    s = text.index(start_marker) + len(start_marker)
+    e = text.index(end_marker, s)
+    return [float(t) for t in re.findall(r"-?\d+\.?\d*(?:[eE]-?\d+)?", text[s:e])]
+
+
+def main():
+    # test/doctest_packing.cpp:21-46 : get_packed_weights of the vector 1..512 (two 16x16 matrices)
+    txt = open(os.path.join(REF, "test/doctest_packing.cpp")).read()
+    vals = numbers_between(txt, "std::vector<float> reference_values = {", "};")
+    assert len(vals) == 512
+    json.dump(
+        {
+            "source": "test/doctest_packing.cpp:21-46",
+            "input_width": 16, "network_width": 16, "output_width": 16, "n_hidden_layers": 1,
+            "unpacked": "1..512",
+            "packed": [int(v) for v in vals],
+        },
+        open(os.path.join(HERE, "packing_16x16x2.json"), "w"),
+    )
+
+    # test/doctest_encodings.cpp:234-285 : 3-D hash grid, x = (1,1,1), params i/(n/2) - 1
+    txt = open(os.path.join(REF, "test/doctest_encodings.cpp")).read()
+    s = txt.index("Test grid encoding using create_grid_encoding instead of factory")
+    vals = numbers_between(txt[s:], "const std::vector<float> reference_out = {", "};")
+    assert len(vals) == 32
+    json.dump(
+        {
+            "source": "test/doctest_encodings.cpp:234-285",
+            "n_dims": 3, "n_levels": 16, "n_features_per_level": 2, "log2_hashmap_size": 19,
+            "base_resolution": 16, "per_level_scale": 2.0, "grid_type": "Hash",
+            "hash": "CoherentPrime", "interpolation": "Linear", "padded_output_width": 32,
+            "input": [1.0, 1.0, 1.0], "params": "i / (n_params / 2) - 1 (test/doctest_encodings.cpp:27-34)",
+            "tolerance": 1.0e-3, "tolerance_metric": "max|a-b| / max(max|a|, max|b|)  (include/common/result_check.h:83-102)",
+            "expected": vals,
+        },
+        open(os.path.join(HERE, "grid_forward_3d.json"), "w"),
+    )
+
+    # toPackedLayoutCoord / fromPackedLayoutCoord point values: test/doctest_common.cpp:25-119
+    json.dump(
+        {
+            "source": "test/doctest_common.cpp:25-119",
+            "to_packed": [[0, 1, 1, 0], [1, 2, 2, 2], [2, 2, 2, 1], [4, 4, 2, 4], [5, 4, 2, 6], [6, 4, 2, 5]],
+            "from_packed": [[0, 1, 1, 0], [1, 2, 2, 2], [2, 2, 2, 1], [4, 4, 2, 4], [5, 4, 2, 6], [6, 4, 2, 5]],
+            "columns": "idx, rows, cols, expected",
+            # test/python/test_packing.py:9-48
+            "pack_4x4": {"unpacked": [[1, 2, 3, 4], [5, 6, 7, 8], [9, 10, 11, 12], [13, 14, 15, 16]],
+                         "packed": [[1, 5, 2, 6], [3, 7, 4, 8], [9, 13, 10, 14], [11, 15, 12, 16]]},
+        },
+        open(os.path.join(HERE, "packed_coords.json"), "w"),
+    )
+
+
+if __name__ == "__main__":
+    main()

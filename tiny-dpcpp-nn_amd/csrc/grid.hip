@@ -1,0 +1,478 @@
+// Multi-resolution hash-grid encoding for gfx950: forward gather + N-linear interpolation,
+// backward scatter-add into an fp32 gradient table.
+//
+// Reference behaviour being reproduced: include/encodings/grid.h:37-135 (kernel_grid),
+// :137-245 (kernel_grid_backward), :588-659 (offset table), :682-694 (zero padding of the output),
+// include/common/common_device.h:700-775 (hashes, grid_index, grid_scale, grid_resolution).
+//
+// One thread owns one point and walks all levels: the coordinates are read once, every corner of a
+// level is gathered before the blend (2^D independent loads in flight), and the whole encoded row is
+// written as contiguous 16-byte pieces. Per-level constants (scale, resolution, table offset, size,
+// how many dimensions enter the dense index, whether the level is hashed) are evaluated once on the
+// host and reach the kernel as scalar kernel arguments; no thread evaluates exp2.
+#include "tnn_internal.h"
+
+#include <cmath>
+#include <cstring>
+
+namespace tnn {
+
+struct GridLevels {
+    uint32_t offset[TNN_GRID_MAX_LEVELS];  // entries
+    uint32_t size[TNN_GRID_MAX_LEVELS];    // entries in the level ("hashmap_size")
+    float scale[TNN_GRID_MAX_LEVELS];
+    uint32_t resolution[TNN_GRID_MAX_LEVELS];
+    // bits 0-3: number of dimensions that enter the strided index; bit 4: level is hashed;
+    // bit 5: size is a power of two
+    uint32_t flags[TNN_GRID_MAX_LEVELS];
+};
+
+struct GridParams {
+    uint32_t n_levels;
+    uint32_t hash_type;
+    uint32_t interpolation;
+    uint32_t padded_width;
+};
+
+// include/common/common_device.h:745-765 evaluated for the loop bounds only: the stride sequence
+// depends on (resolution, size, n_dims) and not on the position.
+static void fill_levels(const tnn_grid_desc *d, GridLevels *lv) {
+    for (uint32_t l = 0; l < d->n_levels; ++l) {
+        const uint32_t size = d->offsets[l + 1] - d->offsets[l];
+        lv->offset[l] = d->offsets[l];
+        lv->size[l] = size;
+        lv->scale[l] = d->scales[l];
+        lv->resolution[l] = d->resolutions[l];
+        uint32_t stride = 1, dims_used = 0;
+        for (uint32_t dim = 0; dim < d->n_dims && stride <= size; ++dim) {
+            ++dims_used;
+            stride *= d->resolutions[l];
+        }
+        const bool hashed = (d->grid_type == TNN_GRID_HASH) && (size < stride);
+        const bool pow2 = (size & (size - 1)) == 0;
+        lv->flags[l] = dims_used | (hashed ? 16u : 0u) | (pow2 ? 32u : 0u);
+    }
+}
+
+template <int D> __device__ __forceinline__ uint32_t hash_pos(const uint32_t (&p)[D], uint32_t hash_type) {
+    // include/common/common_device.h:713-729
+    constexpr uint32_t prime[7] = {1958374283u, 2654435761u, 805459861u, 3674653429u, 2097192037u, 1434869437u, 2165219737u};
+    constexpr uint32_t coherent[7] = {1u, 2654435761u, 805459861u, 3674653429u, 2097192037u, 1434869437u, 2165219737u};
+    constexpr uint32_t reversed[7] = {2165219737u, 1434869437u, 2097192037u, 3674653429u, 805459861u, 2654435761u, 1958374283u};
+    uint32_t r = 0;
+    if (hash_type == TNN_HASH_COHERENT_PRIME) {
+#pragma unroll
+        for (int i = 0; i < D; ++i) r ^= p[i] * coherent[i];
+    } else if (hash_type == TNN_HASH_PRIME) {
+#pragma unroll
+        for (int i = 0; i < D; ++i) r ^= p[i] * prime[i];
+    } else if (hash_type == TNN_HASH_REVERSED_PRIME) {
+#pragma unroll
+        for (int i = 0; i < D; ++i) r ^= p[i] * reversed[i];
+    }
+    return r; // Rng hashes to 0, as in common_device.h:738-740
+}
+
+template <int D>
+__device__ __forceinline__ uint32_t level_index(const uint32_t (&p)[D], uint32_t size, uint32_t res, uint32_t flags,
+                                                uint32_t hash_type) {
+    uint32_t index;
+    if (flags & 16u) {
+        index = hash_pos<D>(p, hash_type);
+    } else {
+        const uint32_t dims_used = flags & 15u;
+        uint32_t stride = 1;
+        index = 0;
+#pragma unroll
+        for (int dim = 0; dim < D; ++dim) {
+            if ((uint32_t)dim < dims_used) {
+                index += p[dim] * stride;
+                stride *= res;
+            }
+        }
+    }
+    if (flags & 32u) return index & (size - 1);
+    return (index >= size) ? index % size : index;
+}
+
+// include/encodings/grid.h:73-93
+template <int D>
+__device__ __forceinline__ void cell_of(const float (&x)[D], float scale, uint32_t interpolation, uint32_t (&cell)[D],
+                                        float (&frac)[D]) {
+#pragma unroll
+    for (int d = 0; d < D; ++d) {
+        float p = __builtin_fmaf(scale, x[d], 0.5f);
+        const float t = floorf(p);
+        cell[d] = (uint32_t)(int)t;
+        p -= t;
+        frac[d] = (interpolation == TNN_INTERP_SMOOTHSTEP) ? p * p * (3.0f - 2.0f * p) : p;
+    }
+}
+
+template <typename P> struct TableVec;
+template <> struct TableVec<float> {
+    static __device__ __forceinline__ float ld(const float *p) { return *p; }
+};
+template <> struct TableVec<fp16_t> {
+    static __device__ __forceinline__ float ld(const fp16_t *p) { return (float)*p; }
+};
+
+template <typename P, int F> __device__ __forceinline__ void load_entry(const P *__restrict__ p, float (&v)[F]) {
+    // F consecutive features of one entry, fetched as a single vector load
+    typedef P vecF __attribute__((ext_vector_type(F)));
+    if (F == 1) {
+        v[0] = (float)p[0];
+    } else {
+        const vecF t = *reinterpret_cast<const vecF *>(p);
+#pragma unroll
+        for (int f = 0; f < F; ++f) v[f] = (float)t[f];
+    }
+}
+
+template <typename O> __device__ __forceinline__ O to_out(float v) { return (O)v; }
+
+constexpr int kGridThreads = 256;
+
+template <int D, int F, typename P, typename O>
+__global__ void __launch_bounds__(kGridThreads)
+    grid_forward_kernel(const GridLevels lv, const GridParams gp, const float *__restrict__ xin, const P *__restrict__ table,
+                        O *__restrict__ out, long long M) {
+    const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= M) return;
+    float x[D];
+#pragma unroll
+    for (int d = 0; d < D; ++d) x[d] = xin[i * D + d];
+    O *orow = out + i * gp.padded_width;
+
+    for (uint32_t l = 0; l < gp.n_levels; ++l) {
+        const uint32_t size = lv.size[l], res = lv.resolution[l], flags = lv.flags[l];
+        const P *g = table + (size_t)lv.offset[l] * F;
+        uint32_t cell[D];
+        float frac[D];
+        cell_of<D>(x, lv.scale[l], gp.interpolation, cell, frac);
+        float result[F];
+        if (gp.interpolation == TNN_INTERP_NEAREST) {
+            const uint32_t idx = level_index<D>(cell, size, res, flags, gp.hash_type);
+            load_entry<P, F>(g + (size_t)idx * F, result);
+        } else {
+            float vals[1 << D][F];
+            float wts[1 << D];
+#pragma unroll
+            for (int c = 0; c < (1 << D); ++c) {
+                float weight = 1.0f;
+                uint32_t loc[D];
+#pragma unroll
+                for (int d = 0; d < D; ++d) {
+                    if ((c & (1 << d)) == 0) {
+                        weight *= 1 - frac[d];
+                        loc[d] = cell[d];
+                    } else {
+                        weight *= frac[d];
+                        loc[d] = cell[d] + 1;
+                    }
+                }
+                wts[c] = weight;
+                const uint32_t idx = level_index<D>(loc, size, res, flags, gp.hash_type);
+                load_entry<P, F>(g + (size_t)idx * F, vals[c]);
+            }
+#pragma unroll
+            for (int f = 0; f < F; ++f) result[f] = 0.0f;
+            // same corner order and fused multiply-add as include/encodings/grid.h:114-129
+#pragma unroll
+            for (int c = 0; c < (1 << D); ++c)
+#pragma unroll
+                for (int f = 0; f < F; ++f) result[f] = __builtin_fmaf(wts[c], vals[c][f], result[f]);
+        }
+#pragma unroll
+        for (int f = 0; f < F; ++f) orow[l * F + f] = to_out<O>(result[f]);
+    }
+    for (uint32_t c = gp.n_levels * F; c < gp.padded_width; ++c) orow[c] = to_out<O>(0.0f);
+}
+
+template <int D>
+__global__ void __launch_bounds__(kGridThreads)
+    grid_indices_kernel(const GridLevels lv, const GridParams gp, const float *__restrict__ xin, uint32_t *__restrict__ out,
+                        long long M) {
+    const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= M) return;
+    float x[D];
+#pragma unroll
+    for (int d = 0; d < D; ++d) x[d] = xin[i * D + d];
+    for (uint32_t l = 0; l < gp.n_levels; ++l) {
+        uint32_t cell[D];
+        float frac[D];
+        cell_of<D>(x, lv.scale[l], gp.interpolation, cell, frac);
+#pragma unroll
+        for (int c = 0; c < (1 << D); ++c) {
+            uint32_t loc[D];
+#pragma unroll
+            for (int d = 0; d < D; ++d) loc[d] = (c & (1 << d)) ? cell[d] + 1 : cell[d];
+            out[(i * gp.n_levels + l) * (1 << D) + c] = level_index<D>(loc, lv.size[l], lv.resolution[l], lv.flags[l], gp.hash_type);
+        }
+    }
+}
+
+// One thread per (point, level): levels are the slow grid dimension so that concurrently running
+// workgroups hit the same level's slice of the gradient table (it stays in L2 while it is hot).
+template <int D, int F, typename G>
+__global__ void __launch_bounds__(kGridThreads)
+    grid_backward_kernel(const GridLevels lv, const GridParams gp, const float *__restrict__ xin, const G *__restrict__ dLdy,
+                         float *__restrict__ grad, long long M) {
+    const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= M) return;
+    const uint32_t l = blockIdx.y;
+    float x[D];
+#pragma unroll
+    for (int d = 0; d < D; ++d) x[d] = xin[i * D + d];
+    float gy[F];
+#pragma unroll
+    for (int f = 0; f < F; ++f) gy[f] = (float)dLdy[i * gp.padded_width + l * F + f];
+
+    const uint32_t size = lv.size[l], res = lv.resolution[l], flags = lv.flags[l];
+    float *g = grad + (size_t)lv.offset[l] * F;
+    uint32_t cell[D];
+    float frac[D];
+    cell_of<D>(x, lv.scale[l], gp.interpolation, cell, frac);
+    if (gp.interpolation == TNN_INTERP_NEAREST) {
+        const uint32_t idx = level_index<D>(cell, size, res, flags, gp.hash_type);
+#pragma unroll
+        for (int f = 0; f < F; ++f) unsafeAtomicAdd(g + (size_t)idx * F + f, gy[f]);
+        return;
+    }
+#pragma unroll
+    for (int c = 0; c < (1 << D); ++c) {
+        float weight = 1.0f;
+        uint32_t loc[D];
+#pragma unroll
+        for (int d = 0; d < D; ++d) {
+            if ((c & (1 << d)) == 0) {
+                weight *= 1 - frac[d];
+                loc[d] = cell[d];
+            } else {
+                weight *= frac[d];
+                loc[d] = cell[d] + 1;
+            }
+        }
+        const uint32_t idx = level_index<D>(loc, size, res, flags, gp.hash_type);
+#pragma unroll
+        for (int f = 0; f < F; ++f) unsafeAtomicAdd(g + (size_t)idx * F + f, weight * gy[f]);
+    }
+}
+
+__global__ void fill_zero_kernel(float4 *__restrict__ p, size_t n4, float *__restrict__ tail, size_t n_tail) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t k = i; k < n4; k += stride) p[k] = float4{0.f, 0.f, 0.f, 0.f};
+    if (i < n_tail) tail[i] = 0.0f;
+}
+
+static int check_grid_desc(const tnn_grid_desc *d) {
+    if (!d) return fail(TNN_ERR_INVALID_ARGUMENT, "desc is NULL");
+    if (d->n_dims != 2 && d->n_dims != 3) return fail(TNN_ERR_UNSUPPORTED, "GridEncoding: n_dims_to_encode %u (2 or 3 are built)", d->n_dims);
+    if (d->n_levels == 0 || d->n_levels > TNN_GRID_MAX_LEVELS)
+        return fail(TNN_ERR_INVALID_ARGUMENT, "GridEncoding: n_levels %u must be at most MAX_N_LEVELS %d", d->n_levels, TNN_GRID_MAX_LEVELS);
+    const uint32_t F = d->n_features_per_level;
+    if (F != 1 && F != 2 && F != 4 && F != 8) return fail(TNN_ERR_INVALID_ARGUMENT, "GridEncoding: n_features_per_level must be 1, 2, 4, or 8.");
+    if (d->param_dtype != TNN_FP32 && d->param_dtype != TNN_FP16) return fail(TNN_ERR_UNSUPPORTED, "table dtype %u", d->param_dtype);
+    if (d->grid_type > TNN_GRID_TILED || d->hash_type > TNN_HASH_RNG || d->interpolation > TNN_INTERP_SMOOTHSTEP)
+        return fail(TNN_ERR_INVALID_ARGUMENT, "invalid grid / hash / interpolation type");
+    return TNN_OK;
+}
+
+template <int D, int F, typename P>
+static int launch_grid_forward_o(const GridLevels &lv, const GridParams &gp, const float *x, const void *table, void *out,
+                                 int out_dtype, size_t M, hipStream_t s) {
+    const unsigned blocks = (unsigned)((M + kGridThreads - 1) / kGridThreads);
+    switch (out_dtype) {
+    case TNN_FP32:
+        hipLaunchKernelGGL((grid_forward_kernel<D, F, P, float>), dim3(blocks), dim3(kGridThreads), 0, s, lv, gp, x, (const P *)table,
+                           (float *)out, (long long)M);
+        break;
+    case TNN_BF16:
+        hipLaunchKernelGGL((grid_forward_kernel<D, F, P, bf16_t>), dim3(blocks), dim3(kGridThreads), 0, s, lv, gp, x, (const P *)table,
+                           (bf16_t *)out, (long long)M);
+        break;
+    case TNN_FP16:
+        hipLaunchKernelGGL((grid_forward_kernel<D, F, P, fp16_t>), dim3(blocks), dim3(kGridThreads), 0, s, lv, gp, x, (const P *)table,
+                           (fp16_t *)out, (long long)M);
+        break;
+    default: return fail(TNN_ERR_UNSUPPORTED, "out_dtype %d", out_dtype);
+    }
+    return check_launch("grid_forward_kernel");
+}
+
+template <int D, int F>
+static int launch_grid_forward_p(const tnn_grid_desc *d, const GridLevels &lv, const GridParams &gp, const float *x,
+                                 const void *table, void *out, int out_dtype, size_t M, hipStream_t s) {
+    if (d->param_dtype == TNN_FP32) return launch_grid_forward_o<D, F, float>(lv, gp, x, table, out, out_dtype, M, s);
+    return launch_grid_forward_o<D, F, fp16_t>(lv, gp, x, table, out, out_dtype, M, s);
+}
+
+template <int D, int F>
+static int launch_grid_backward_g(const GridLevels &lv, const GridParams &gp, const float *x, const void *dLdy, int dy_dtype,
+                                  float *grad, size_t M, hipStream_t s) {
+    const dim3 grid((unsigned)((M + kGridThreads - 1) / kGridThreads), gp.n_levels);
+    switch (dy_dtype) {
+    case TNN_FP32:
+        hipLaunchKernelGGL((grid_backward_kernel<D, F, float>), grid, dim3(kGridThreads), 0, s, lv, gp, x, (const float *)dLdy, grad,
+                           (long long)M);
+        break;
+    case TNN_BF16:
+        hipLaunchKernelGGL((grid_backward_kernel<D, F, bf16_t>), grid, dim3(kGridThreads), 0, s, lv, gp, x, (const bf16_t *)dLdy, grad,
+                           (long long)M);
+        break;
+    case TNN_FP16:
+        hipLaunchKernelGGL((grid_backward_kernel<D, F, fp16_t>), grid, dim3(kGridThreads), 0, s, lv, gp, x, (const fp16_t *)dLdy, grad,
+                           (long long)M);
+        break;
+    default: return fail(TNN_ERR_UNSUPPORTED, "dy_dtype %d", dy_dtype);
+    }
+    return check_launch("grid_backward_kernel");
+}
+
+#define TNN_DISPATCH_DF(desc, CALL)                                                              \
+    do {                                                                                         \
+        const uint32_t F__ = (desc)->n_features_per_level;                                       \
+        if ((desc)->n_dims == 2) {                                                               \
+            constexpr int D_ = 2;                                                                \
+            if (F__ == 1) { constexpr int F_ = 1; CALL; }                                        \
+            else if (F__ == 2) { constexpr int F_ = 2; CALL; }                                   \
+            else if (F__ == 4) { constexpr int F_ = 4; CALL; }                                   \
+            else { constexpr int F_ = 8; CALL; }                                                 \
+        } else {                                                                                 \
+            constexpr int D_ = 3;                                                                \
+            if (F__ == 1) { constexpr int F_ = 1; CALL; }                                        \
+            else if (F__ == 2) { constexpr int F_ = 2; CALL; }                                   \
+            else if (F__ == 4) { constexpr int F_ = 4; CALL; }                                   \
+            else { constexpr int F_ = 8; CALL; }                                                 \
+        }                                                                                        \
+    } while (0)
+
+} // namespace tnn
+
+using namespace tnn;
+
+TNN_API int tnn_grid_desc_init(tnn_grid_desc *desc, uint32_t n_dims, uint32_t n_levels, uint32_t n_features_per_level,
+                               uint32_t log2_hashmap_size, uint32_t base_resolution, float per_level_scale,
+                               uint32_t grid_type, uint32_t hash_type, uint32_t interpolation, uint32_t param_dtype) {
+    if (!desc) return fail(TNN_ERR_INVALID_ARGUMENT, "desc is NULL");
+    memset(desc, 0, sizeof(*desc));
+    desc->n_dims = n_dims;
+    desc->n_levels = n_levels;
+    desc->n_features_per_level = n_features_per_level;
+    desc->log2_hashmap_size = log2_hashmap_size;
+    desc->base_resolution = base_resolution;
+    desc->per_level_scale = per_level_scale;
+    desc->grid_type = grid_type;
+    desc->hash_type = hash_type;
+    desc->interpolation = interpolation;
+    desc->param_dtype = param_dtype;
+    int rc = check_grid_desc(desc);
+    if (rc) return rc;
+    if (log2_hashmap_size > 31) return fail(TNN_ERR_INVALID_ARGUMENT, "log2_hashmap_size %u", log2_hashmap_size);
+    if (base_resolution == 0 || !(per_level_scale > 0.0f)) return fail(TNN_ERR_INVALID_ARGUMENT, "base_resolution / per_level_scale");
+
+    // include/encodings/grid.h:604-644 with grid_scale / grid_resolution (common_device.h:767-775)
+    const float log2_pls = std::log2(per_level_scale);
+    uint64_t offset = 0;
+    for (uint32_t i = 0; i < n_levels; ++i) {
+        const float scale = std::exp2((float)i * log2_pls) * (float)base_resolution - 1.0f;
+        const uint32_t resolution = (uint32_t)std::ceil(scale) + 1u;
+        const uint32_t max_params = UINT32_MAX / 2;
+        uint32_t params_in_level;
+        if (std::pow((float)resolution, (float)n_dims) > (float)max_params) {
+            params_in_level = max_params;
+        } else {
+            params_in_level = 1;
+            for (uint32_t k = 0; k < n_dims; ++k) params_in_level *= resolution;
+        }
+        params_in_level = (params_in_level + 7u) / 8u * 8u;
+        if (grid_type == TNN_GRID_TILED) {
+            uint32_t t = 1;
+            for (uint32_t k = 0; k < n_dims; ++k) t *= base_resolution;
+            if (t < params_in_level) params_in_level = t;
+        } else if (grid_type == TNN_GRID_HASH) {
+            const uint32_t t = 1u << log2_hashmap_size;
+            if (t < params_in_level) params_in_level = t;
+        }
+        desc->offsets[i] = (uint32_t)offset;
+        desc->scales[i] = scale;
+        desc->resolutions[i] = resolution;
+        offset += params_in_level;
+        if (offset > UINT32_MAX) return fail(TNN_ERR_INVALID_ARGUMENT, "grid table exceeds 2^32 entries");
+    }
+    desc->offsets[n_levels] = (uint32_t)offset;
+    return TNN_OK;
+}
+
+TNN_API size_t tnn_grid_n_params(const tnn_grid_desc *desc) {
+    if (check_grid_desc(desc)) return 0;
+    return (size_t)desc->offsets[desc->n_levels] * desc->n_features_per_level;
+}
+
+static int grid_common(const tnn_grid_desc *desc, uint32_t padded_width, size_t M, GridLevels *lv, GridParams *gp) {
+    int rc = check_grid_desc(desc);
+    if (rc) return rc;
+    // include/encodings/grid.h:665-677
+    if (padded_width == 0) return fail(TNN_ERR_INVALID_ARGUMENT, "Can't have width == 0");
+    if (padded_width < desc->n_levels * desc->n_features_per_level)
+        return fail(TNN_ERR_INVALID_ARGUMENT, "Dimension mismatch grid encoding output: padded width %u < %u features", padded_width,
+                    desc->n_levels * desc->n_features_per_level);
+    if (M == 0) return fail(TNN_ERR_INVALID_ARGUMENT, "batch_size == 0");
+    if (M > 0x7fffffffull * kGridThreads) return fail(TNN_ERR_INVALID_ARGUMENT, "batch too large");
+    fill_levels(desc, lv);
+    gp->n_levels = desc->n_levels;
+    gp->hash_type = desc->hash_type;
+    gp->interpolation = desc->interpolation;
+    gp->padded_width = padded_width;
+    return TNN_OK;
+}
+
+TNN_API int tnn_grid_forward(const tnn_grid_desc *desc, const float *d_x, const void *d_table, void *d_out, int out_dtype,
+                             uint32_t padded_width, size_t M, tnn_stream_t stream) {
+    GridLevels lv;
+    GridParams gp;
+    int rc = grid_common(desc, padded_width, M, &lv, &gp);
+    if (rc) return rc;
+    if (!d_x || !d_table || !d_out) return fail(TNN_ERR_INVALID_ARGUMENT, "NULL pointer argument");
+    TNN_DISPATCH_DF(desc, rc = (launch_grid_forward_p<D_, F_>(desc, lv, gp, d_x, d_table, d_out, out_dtype, M, as_stream(stream))));
+    return rc;
+}
+
+TNN_API int tnn_grid_backward(const tnn_grid_desc *desc, const float *d_x, const void *d_dLdy, int dy_dtype,
+                              uint32_t padded_width, float *d_grad_table, int overwrite, size_t M, tnn_stream_t stream) {
+    GridLevels lv;
+    GridParams gp;
+    int rc = grid_common(desc, padded_width, M, &lv, &gp);
+    if (rc) return rc;
+    if (!d_x || !d_dLdy || !d_grad_table) return fail(TNN_ERR_INVALID_ARGUMENT, "NULL pointer argument");
+    hipStream_t s = as_stream(stream);
+    if (overwrite) {
+        // a fill kernel rather than a memset node, so the call can be captured into a HIP graph
+        const size_t n = tnn_grid_n_params(desc);
+        if (reinterpret_cast<uintptr_t>(d_grad_table) & 15) return fail(TNN_ERR_INVALID_ARGUMENT, "d_grad_table must be 16-byte aligned");
+        const size_t n4 = n / 4;
+        const size_t n_tail = n - n4 * 4;
+        size_t blocks = (n4 + 255) / 256;
+        if (blocks > 4096) blocks = 4096;
+        if (blocks < 4) blocks = 4;
+        hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)blocks), dim3(256), 0, s, (float4 *)d_grad_table, n4, d_grad_table + n4 * 4, n_tail);
+        if ((rc = check_launch("fill_zero_kernel"))) return rc;
+    }
+    TNN_DISPATCH_DF(desc, rc = (launch_grid_backward_g<D_, F_>(lv, gp, d_x, d_dLdy, dy_dtype, d_grad_table, M, s)));
+    return rc;
+}
+
+TNN_API int tnn_grid_indices(const tnn_grid_desc *desc, const float *d_x, uint32_t *d_indices, size_t M, tnn_stream_t stream) {
+    GridLevels lv;
+    GridParams gp;
+    int rc = grid_common(desc, desc ? desc->n_levels * desc->n_features_per_level : 0, M, &lv, &gp);
+    if (rc) return rc;
+    if (!d_x || !d_indices) return fail(TNN_ERR_INVALID_ARGUMENT, "NULL pointer argument");
+    const unsigned blocks = (unsigned)((M + kGridThreads - 1) / kGridThreads);
+    if (desc->n_dims == 2)
+        hipLaunchKernelGGL((grid_indices_kernel<2>), dim3(blocks), dim3(kGridThreads), 0, as_stream(stream), lv, gp, d_x, d_indices, (long long)M);
+    else
+        hipLaunchKernelGGL((grid_indices_kernel<3>), dim3(blocks), dim3(kGridThreads), 0, as_stream(stream), lv, gp, d_x, d_indices, (long long)M);
+    return check_launch("grid_indices_kernel");
+}

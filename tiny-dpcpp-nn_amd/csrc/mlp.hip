@@ -1,0 +1,642 @@
+// Fully fused MLP for gfx950: inference, training forward, fused backward (delta propagation),
+// weight gradients. One wave streams a tile of 32 batch rows through every layer:
+//   * the transposed product  Y^T = W^T * X^T  is evaluated with v_mfma_f32_32x32x16_{bf16,f16}:
+//     the weights are the A operand (staged once per workgroup in LDS, already in operand order),
+//     the activations are the B operand and never leave the registers between layers;
+//   * lane (j = lane % 32, h = lane / 32) owns batch row j of the tile; for every block of 16
+//     features it holds the 8 features 16*kb + 8*h + [0, 8), i.e. one aligned 16-byte piece of the
+//     row-major row. Loads, stores and MFMA B operands all use that same register layout.
+//
+// Reference behaviour being reproduced: include/network/kernel_esimd.h:565-640 (forward /
+// inference), :160-228 (delta propagation), :230-239 (dW = delta^T * a), rounding points
+// :443-487 (fp32 accumulate -> round to T -> activation; backward mask / sigmoid slope applied to
+// the fp32 accumulator before rounding).
+#include "tnn_internal.h"
+
+namespace tnn {
+
+constexpr int kFwdThreads = 512; // 8 waves per workgroup share one LDS copy of the weights
+constexpr int kWaveSize = 64;
+
+// ------------------------------------------------------------------------------------------
+// Operand preparation
+// ------------------------------------------------------------------------------------------
+
+// Operand order ("prepared" layout), per weight matrix l, per 32-row output tile a, per 16-deep
+// contraction block kb: 64 lanes x 8 elements, lane = 32*h + i, element t:
+//   forward : W_l[k = 16*kb + 8*h + t][n = 32*a + swap23(i)]
+//   backward: W_l[k = 32*a + swap23(i)][n = 16*kb + 8*h + t]      (the product with W_l^T)
+// Rows beyond the width (only for width 16, whose single tile is half empty) are zero.
+template <typename T, typename SRC>
+__global__ void prepare_weights_kernel(const SRC *__restrict__ packed, T *__restrict__ fwd, T *__restrict__ bwd, int W,
+                                       int n_mats) {
+    const int NI = (W + 31) / 32, NK = W / 16;
+    const int per_mat = NI * NK * 512;
+    const int total = n_mats * per_mat;
+    for (int idx = blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += gridDim.x * blockDim.x) {
+        const int l = idx / per_mat;
+        int r = idx % per_mat;
+        const int t = r & 7;
+        const int lane = (r >> 3) & 63;
+        r >>= 9;
+        const int kb = r % NK, a = r / NK;
+        const int h = lane >> 5, i = lane & 31;
+        const int outer = 32 * a + swap23(i);  // output feature of the product
+        const int inner = 16 * kb + 8 * h + t; // contraction index
+        const SRC *src = packed + (size_t)l * W * W;
+        T vf = (T)0.0f, vb = (T)0.0f;
+        if (outer < W) {
+            vf = (T)(float)src[packed_coord(inner, outer, W)]; // W[k = inner][n = outer]
+            vb = (T)(float)src[packed_coord(outer, inner, W)]; // W[k = outer][n = inner]
+        }
+        if (fwd) fwd[idx] = vf;
+        if (bwd) bwd[idx] = vb;
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+// Device helpers
+// ------------------------------------------------------------------------------------------
+
+template <int ACT> __device__ __forceinline__ float act_f32(float v) {
+    if (ACT == TNN_ACT_RELU) return fmaxf(v, 0.0f);
+    if (ACT == TNN_ACT_SIGMOID) return __builtin_amdgcn_rcpf(1.0f + __expf(-v));
+    return v;
+}
+
+// Accumulator half (8 fp32 of one 32x32 tile) -> activation -> 8 values of T.
+// ReLU before or after the rounding gives the same value (rounding keeps the sign).
+template <typename T, int ACT, int HALF>
+__device__ __forceinline__ typename Storage<T>::vec8 act_convert(const f32x16 &c) {
+    f32x8 v;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = act_f32<ACT>(c[HALF * 8 + e]);
+    return __builtin_convertvector(v, typename Storage<T>::vec8);
+}
+
+// Backward: fp32 accumulator, masked / scaled by the stored forward activation, then rounded.
+template <typename T, int ACT, int HALF>
+__device__ __forceinline__ typename Storage<T>::vec8 bwd_convert(const f32x16 &c,
+                                                                 const typename Storage<T>::vec8 &fwd) {
+    f32x8 v;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        float t = c[HALF * 8 + e];
+        const float f = (float)fwd[e];
+        if (ACT == TNN_ACT_RELU) t = (f <= 0.0f) ? 0.0f : t;
+        if (ACT == TNN_ACT_SIGMOID) t = t * (f * (1.0f - f));
+        v[e] = t;
+    }
+    return __builtin_convertvector(v, typename Storage<T>::vec8);
+}
+
+template <typename T, int W> struct Tile {
+    static constexpr int NK = W / 16;
+    static constexpr int NI = (W + 31) / 32;
+    typedef typename Storage<T>::vec8 vec8;
+
+    // Row-major row `row` of an M x W matrix -> the lane's NK 16-byte pieces.
+    static __device__ __forceinline__ void load(vec8 (&r)[NK], const T *__restrict__ base, long long row, int h,
+                                                bool valid) {
+        const vec8 *p = reinterpret_cast<const vec8 *>(base + row * W) + h;
+#pragma unroll
+        for (int kb = 0; kb < NK; ++kb) {
+            if (valid)
+                r[kb] = p[2 * kb];
+            else
+                r[kb] = vec8{};
+        }
+    }
+    static __device__ __forceinline__ void store(const vec8 (&r)[NK], T *__restrict__ base, long long row, int h,
+                                                 bool valid) {
+        vec8 *p = reinterpret_cast<vec8 *>(base + row * W) + h;
+        if (valid) {
+#pragma unroll
+            for (int kb = 0; kb < NK; ++kb) p[2 * kb] = r[kb];
+        }
+    }
+
+    // acc[a] = sum_kb frag(l, a, kb) * b[kb]
+    template <bool W_IN_LDS>
+    static __device__ __forceinline__ void matmul(f32x16 (&acc)[NI], const vec8 (&b)[NK], const vec8 *__restrict__ lds_w,
+                                                  const vec8 *__restrict__ glb_w, int l, int lane) {
+        const vec8 *w = (W_IN_LDS ? lds_w : glb_w) + (size_t)l * (NI * NK * kWaveSize) + lane;
+#pragma unroll
+        for (int a = 0; a < NI; ++a) acc[a] = f32x16{};
+#pragma unroll
+        for (int kb = 0; kb < NK; ++kb) {
+#pragma unroll
+            for (int a = 0; a < NI; ++a) {
+                const vec8 frag = w[(a * NK + kb) * kWaveSize];
+                acc[a] = Storage<T>::mfma(frag, b[kb], acc[a]);
+            }
+        }
+    }
+
+    template <int ACT> static __device__ __forceinline__ void repack(vec8 (&r)[NK], const f32x16 (&acc)[NI]) {
+#pragma unroll
+        for (int a = 0; a < NI; ++a) {
+            r[2 * a] = act_convert<T, ACT, 0>(acc[a]);
+            if (2 * a + 1 < NK) r[2 * a + 1] = act_convert<T, ACT, 1>(acc[a]);
+        }
+    }
+    static __device__ __forceinline__ void repack_rt(vec8 (&r)[NK], const f32x16 (&acc)[NI], int act) {
+        if (act == TNN_ACT_RELU)
+            repack<TNN_ACT_RELU>(r, acc);
+        else if (act == TNN_ACT_SIGMOID)
+            repack<TNN_ACT_SIGMOID>(r, acc);
+        else
+            repack<TNN_ACT_NONE>(r, acc);
+    }
+
+    template <int ACT>
+    static __device__ __forceinline__ void bwd_repack(vec8 (&r)[NK], const f32x16 (&acc)[NI], const vec8 (&fwd)[NK]) {
+#pragma unroll
+        for (int a = 0; a < NI; ++a) {
+            r[2 * a] = bwd_convert<T, ACT, 0>(acc[a], fwd[2 * a]);
+            if (2 * a + 1 < NK) r[2 * a + 1] = bwd_convert<T, ACT, 1>(acc[a], fwd[2 * a + 1 < NK ? 2 * a + 1 : 0]);
+        }
+    }
+};
+
+template <typename T, int W>
+__device__ __forceinline__ void stage_weights(typename Storage<T>::vec8 *lds_w,
+                                              const typename Storage<T>::vec8 *__restrict__ glb_w, int n_mats) {
+    constexpr int per_mat = Tile<T, W>::NI * Tile<T, W>::NK * kWaveSize;
+    const int n = n_mats * per_mat;
+    for (int f = threadIdx.x; f < n; f += blockDim.x) lds_w[f] = glb_w[f];
+    __syncthreads();
+}
+
+// ------------------------------------------------------------------------------------------
+// Forward / inference
+// ------------------------------------------------------------------------------------------
+// out: STORE_INTERM ? (n_mats + 1) matrices M x W ([0] = copy of x) : one matrix M x W.
+template <typename T, int W, bool STORE_INTERM, bool W_IN_LDS>
+__global__ void __launch_bounds__(kFwdThreads)
+    mlp_forward_kernel(const typename Storage<T>::vec8 *__restrict__ wprep, const T *__restrict__ x, T *__restrict__ out,
+                       int n_mats, int act, int out_act, long long M) {
+    typedef Tile<T, W> TL;
+    typedef typename Storage<T>::vec8 vec8;
+    constexpr int NK = TL::NK, NI = TL::NI;
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+    vec8 *lds_w = reinterpret_cast<vec8 *>(smem_raw);
+    if (W_IN_LDS) stage_weights<T, W>(lds_w, wprep, n_mats);
+
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int j = lane & 31, h = lane >> 5;
+    const long long n_tiles = (M + 31) / 32;
+    const long long stride = (long long)gridDim.x * (blockDim.x >> 6);
+    long long tile = (long long)blockIdx.x * (blockDim.x >> 6) + wave;
+
+    vec8 cur[NK];
+    if (tile < n_tiles) TL::load(cur, x, tile * 32 + j, h, tile * 32 + j < M);
+    while (tile < n_tiles) {
+        const long long row = tile * 32 + j;
+        const bool valid = row < M;
+        // prefetch the next tile of this wave while the current one is being computed
+        const long long next_tile = tile + stride;
+        vec8 nxt[NK];
+        if (next_tile < n_tiles) TL::load(nxt, x, next_tile * 32 + j, h, next_tile * 32 + j < M);
+
+        if (STORE_INTERM) TL::store(cur, out, row, h, valid);
+        f32x16 acc[NI];
+        for (int l = 0; l < n_mats - 1; ++l) {
+            TL::template matmul<W_IN_LDS>(acc, cur, lds_w, wprep, l, lane);
+            TL::repack_rt(cur, acc, act);
+            if (STORE_INTERM) TL::store(cur, out + (size_t)(l + 1) * M * W, row, h, valid);
+        }
+        TL::template matmul<W_IN_LDS>(acc, cur, lds_w, wprep, n_mats - 1, lane);
+        TL::repack_rt(cur, acc, out_act);
+        TL::store(cur, STORE_INTERM ? out + (size_t)n_mats * M * W : out, row, h, valid);
+
+        if (next_tile < n_tiles) {
+#pragma unroll
+            for (int kb = 0; kb < NK; ++kb) cur[kb] = nxt[kb];
+        }
+        tile = next_tile;
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+// Backward: delta propagation (include/network/kernel_esimd.h:186-227)
+// ------------------------------------------------------------------------------------------
+template <typename T, int W, bool W_IN_LDS>
+__global__ void __launch_bounds__(kFwdThreads)
+    mlp_backward_kernel(const typename Storage<T>::vec8 *__restrict__ wprep_bwd, const T *__restrict__ dLdy,
+                        const T *__restrict__ interm_fwd, T *__restrict__ interm_bwd, T *__restrict__ dLdx, int n_mats,
+                        int act, int out_act, long long M) {
+    typedef Tile<T, W> TL;
+    typedef typename Storage<T>::vec8 vec8;
+    constexpr int NK = TL::NK, NI = TL::NI;
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+    vec8 *lds_w = reinterpret_cast<vec8 *>(smem_raw);
+    if (W_IN_LDS) stage_weights<T, W>(lds_w, wprep_bwd, n_mats);
+
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int j = lane & 31, h = lane >> 5;
+    const long long n_tiles = (M + 31) / 32;
+    const long long stride = (long long)gridDim.x * (blockDim.x >> 6);
+    const size_t mat = (size_t)M * W;
+
+    for (long long tile = (long long)blockIdx.x * (blockDim.x >> 6) + wave; tile < n_tiles; tile += stride) {
+        const long long row = tile * 32 + j;
+        const bool valid = row < M;
+        vec8 cur[NK], fwd[NK];
+        TL::load(cur, dLdy, row, h, valid);
+        // derivative of the output activation, applied on the T tile (kernel_esimd.h:193-201)
+        if (out_act != TNN_ACT_NONE) {
+            TL::load(fwd, interm_fwd + (size_t)n_mats * mat, row, h, valid);
+#pragma unroll
+            for (int kb = 0; kb < NK; ++kb) {
+                f32x8 v;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const float g = (float)cur[kb][e], f = (float)fwd[kb][e];
+                    v[e] = (out_act == TNN_ACT_RELU) ? ((f <= 0.0f) ? 0.0f : g) : g * (f * (1.0f - f));
+                }
+                cur[kb] = __builtin_convertvector(v, vec8);
+            }
+        }
+        if (interm_bwd) TL::store(cur, interm_bwd + (size_t)(n_mats - 1) * mat, row, h, valid);
+
+        f32x16 acc[NI];
+        for (int l = n_mats - 1; l > 0; --l) {
+            // the forward activation of layer l-1 that gates delta_{l-1}; issued before the MFMAs
+            if (act != TNN_ACT_NONE) TL::load(fwd, interm_fwd + (size_t)l * mat, row, h, valid);
+            TL::template matmul<W_IN_LDS>(acc, cur, lds_w, wprep_bwd, l, lane);
+            if (act == TNN_ACT_RELU)
+                TL::template bwd_repack<TNN_ACT_RELU>(cur, acc, fwd);
+            else if (act == TNN_ACT_SIGMOID)
+                TL::template bwd_repack<TNN_ACT_SIGMOID>(cur, acc, fwd);
+            else
+                TL::template repack<TNN_ACT_NONE>(cur, acc);
+            if (interm_bwd) TL::store(cur, interm_bwd + (size_t)(l - 1) * mat, row, h, valid);
+        }
+        if (dLdx) {
+            TL::template matmul<W_IN_LDS>(acc, cur, lds_w, wprep_bwd, 0, lane);
+            TL::template repack<TNN_ACT_NONE>(cur, acc);
+            TL::store(cur, dLdx, row, h, valid);
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+// Weight gradients: dW_l[n][k] = sum_m delta_l[m][n] * a_l[m][k]   (kernel_esimd.h:230-239)
+// ------------------------------------------------------------------------------------------
+constexpr int kDwThreads = 256;
+constexpr int kDwSlab = 64; // rows staged in LDS per step
+
+// Contraction runs over batch rows, which the streaming kernels keep one-per-lane; both operands are
+// therefore transposed through LDS: a slab of rows is stored row-major and read back column-wise.
+// Workgroup (l, c) reduces rows [c*rows_per_chunk, (c+1)*rows_per_chunk) of matrix l into one (or, for
+// W <= 32, four) fp32 partial W x W tiles in the workspace; dw_reduce_kernel sums the partials.
+template <typename T, int W>
+__global__ void __launch_bounds__(kDwThreads)
+    mlp_dw_partial_kernel(const T *__restrict__ interm_bwd, const T *__restrict__ interm_fwd, float *__restrict__ partials,
+                          int n_mats, long long M, long long rows_per_chunk) {
+    typedef typename Storage<T>::vec8 vec8;
+    constexpr int NI = (W + 31) / 32;
+    constexpr int PITCH = W + 8;                 // elements; keeps 16-byte alignment, skews banks
+    constexpr int TILES = NI * NI;
+    constexpr int TPW = (TILES + 3) / 4;         // tiles per wave (W=128: 4, W=64: 1, else 1)
+    constexpr bool SPLIT_ROWS = (TILES == 1);    // W <= 32: waves split the rows of a slab instead
+    __shared__ __attribute__((aligned(16))) T lds_d[kDwSlab * PITCH];
+    __shared__ __attribute__((aligned(16))) T lds_a[kDwSlab * PITCH];
+
+    const int l = blockIdx.y;
+    const long long chunk = blockIdx.x;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int i = lane & 31, h = lane >> 5;
+    const T *dmat = interm_bwd + (size_t)l * M * W;
+    const T *amat = interm_fwd + (size_t)l * M * W;
+    const long long row0 = chunk * rows_per_chunk;
+    long long row_end = row0 + rows_per_chunk;
+    if (row_end > M) row_end = M;
+
+    f32x16 acc[TPW];
+#pragma unroll
+    for (int t = 0; t < TPW; ++t) acc[t] = f32x16{};
+
+    constexpr int CHUNKS_PER_ROW = W / 8;
+    for (long long slab = row0; slab < row_end; slab += kDwSlab) {
+        __syncthreads();
+        for (int c = threadIdx.x; c < kDwSlab * CHUNKS_PER_ROW; c += kDwThreads) {
+            const int r = c / CHUNKS_PER_ROW, cc = c % CHUNKS_PER_ROW;
+            const long long row = slab + r;
+            vec8 dv = vec8{}, av = vec8{};
+            if (row < row_end) {
+                dv = reinterpret_cast<const vec8 *>(dmat + row * W)[cc];
+                av = reinterpret_cast<const vec8 *>(amat + row * W)[cc];
+            }
+            *reinterpret_cast<vec8 *>(&lds_d[r * PITCH + cc * 8]) = dv;
+            *reinterpret_cast<vec8 *>(&lds_a[r * PITCH + cc * 8]) = av;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int kb = 0; kb < kDwSlab / 16; ++kb) {
+            if (SPLIT_ROWS && kb != wave) continue;
+            const int rbase = 16 * kb + 8 * h;
+            if (SPLIT_ROWS) {
+                vec8 A = vec8{}, B = vec8{};
+                if (i < W) {
+#pragma unroll
+                    for (int t = 0; t < 8; ++t) {
+                        A[t] = lds_d[(rbase + t) * PITCH + i];
+                        B[t] = lds_a[(rbase + t) * PITCH + i];
+                    }
+                }
+                acc[0] = Storage<T>::mfma(A, B, acc[0]);
+            } else {
+                // wave owns tiles (a, b): W=64 -> a = wave/2, b = wave%2 ; W=128 -> a = wave, b = 0..3
+                const int a = (NI == 2) ? (wave >> 1) : wave;
+                vec8 A;
+#pragma unroll
+                for (int t = 0; t < 8; ++t) A[t] = lds_d[(rbase + t) * PITCH + 32 * a + i];
+#pragma unroll
+                for (int tt = 0; tt < TPW; ++tt) {
+                    const int b = (NI == 2) ? (wave & 1) : tt;
+                    vec8 B;
+#pragma unroll
+                    for (int t = 0; t < 8; ++t) B[t] = lds_a[(rbase + t) * PITCH + 32 * b + i];
+                    acc[tt] = Storage<T>::mfma(A, B, acc[tt]);
+                }
+            }
+        }
+    }
+    // accumulator register r of lane (j = i, h) is element (row 8*(r/4) + 4*h + r%4, column j) of the tile
+    const int ppw = SPLIT_ROWS ? 4 : 1;
+    float *out = partials + (((size_t)chunk * ppw + (SPLIT_ROWS ? wave : 0)) * n_mats + l) * W * W;
+#pragma unroll
+    for (int tt = 0; tt < TPW; ++tt) {
+        const int a = SPLIT_ROWS ? 0 : ((NI == 2) ? (wave >> 1) : wave);
+        const int b = SPLIT_ROWS ? 0 : ((NI == 2) ? (wave & 1) : tt);
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int n = 32 * a + 8 * (r >> 2) + 4 * h + (r & 3);
+            const int k = 32 * b + i;
+            if (n < W && k < W) out[n * W + k] = acc[tt][r];
+        }
+    }
+}
+
+template <typename T>
+__global__ void dw_reduce_kernel(const float *__restrict__ partials, int n_partials, int n_elems, T *__restrict__ dW_T,
+                                 float *__restrict__ dW_f32) {
+    const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= n_elems) return;
+    float s = 0.0f;
+    for (int p = 0; p < n_partials; ++p) s += partials[(size_t)p * n_elems + idx];
+    if (dW_f32)
+        dW_f32[idx] = s;
+    else
+        dW_T[idx] = (T)s;
+}
+
+// ------------------------------------------------------------------------------------------
+// Host side
+// ------------------------------------------------------------------------------------------
+struct DeviceInfo {
+    int n_cu = 0;
+    size_t max_lds = 0;
+    bool ok = false;
+};
+
+static const DeviceInfo &device_info() {
+    static thread_local DeviceInfo info[16];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 16) {
+        static DeviceInfo bad;
+        return bad;
+    }
+    if (!info[dev].ok) {
+        hipDeviceProp_t p;
+        if (hipGetDeviceProperties(&p, dev) == hipSuccess) {
+            info[dev].n_cu = p.multiProcessorCount;
+            info[dev].max_lds = p.maxSharedMemoryPerMultiProcessor ? p.maxSharedMemoryPerMultiProcessor : p.sharedMemPerBlock;
+            info[dev].ok = true;
+        }
+    }
+    return info[dev];
+}
+
+static size_t prepared_elems(const tnn_mlp_desc *d) {
+    const int W = d->width, NI = (W + 31) / 32, NK = W / 16;
+    return (size_t)(d->n_hidden_layers + 1) * NI * NK * 512;
+}
+
+// LDS the weights may take and still leave room for two workgroups per CU.
+constexpr size_t kLdsBudget = 144 * 1024;
+
+template <typename T, int W, bool STORE_INTERM>
+static int launch_forward(const tnn_mlp_desc *d, const void *wprep, const void *x, void *out, size_t M, hipStream_t s) {
+    typedef typename Storage<T>::vec8 vec8;
+    const int n_mats = d->n_hidden_layers + 1;
+    const size_t wbytes = prepared_elems(d) * sizeof(T);
+    const DeviceInfo &di = device_info();
+    if (!di.ok) return fail(TNN_ERR_HIP, "no usable HIP device");
+    const long long n_tiles = ((long long)M + 31) / 32;
+    const int waves = kFwdThreads / 64;
+    long long blocks = (n_tiles + waves - 1) / waves;
+    const bool in_lds = wbytes <= kLdsBudget;
+    const int per_cu = (in_lds && wbytes > 72 * 1024) ? 1 : 2;
+    if (blocks > (long long)di.n_cu * per_cu) blocks = (long long)di.n_cu * per_cu;
+    if (blocks < 1) blocks = 1;
+    if (in_lds) {
+        auto k = mlp_forward_kernel<T, W, STORE_INTERM, true>;
+        if (wbytes > 48 * 1024 &&
+            hipFuncSetAttribute(reinterpret_cast<const void *>(k), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                (int)wbytes) != hipSuccess)
+            return fail(TNN_ERR_HIP, "cannot reserve %zu bytes of LDS", wbytes);
+        hipLaunchKernelGGL(k, dim3((unsigned)blocks), dim3(kFwdThreads), wbytes, s, (const vec8 *)wprep, (const T *)x,
+                           (T *)out, n_mats, d->activation, d->output_activation, (long long)M);
+    } else {
+        hipLaunchKernelGGL((mlp_forward_kernel<T, W, STORE_INTERM, false>), dim3((unsigned)blocks), dim3(kFwdThreads), 0,
+                           s, (const vec8 *)wprep, (const T *)x, (T *)out, n_mats, d->activation, d->output_activation,
+                           (long long)M);
+    }
+    return check_launch("mlp_forward_kernel");
+}
+
+template <typename T, int W>
+static int launch_backward(const tnn_mlp_desc *d, const void *wprep_bwd, const void *dLdy, const void *interm_fwd,
+                           void *interm_bwd, void *dLdx, size_t M, hipStream_t s) {
+    typedef typename Storage<T>::vec8 vec8;
+    const int n_mats = d->n_hidden_layers + 1;
+    const size_t wbytes = prepared_elems(d) * sizeof(T);
+    const DeviceInfo &di = device_info();
+    if (!di.ok) return fail(TNN_ERR_HIP, "no usable HIP device");
+    const long long n_tiles = ((long long)M + 31) / 32;
+    const int waves = kFwdThreads / 64;
+    long long blocks = (n_tiles + waves - 1) / waves;
+    const bool in_lds = wbytes <= kLdsBudget;
+    const int per_cu = (in_lds && wbytes > 72 * 1024) ? 1 : 2;
+    if (blocks > (long long)di.n_cu * per_cu) blocks = (long long)di.n_cu * per_cu;
+    if (blocks < 1) blocks = 1;
+    if (in_lds) {
+        auto k = mlp_backward_kernel<T, W, true>;
+        if (wbytes > 48 * 1024 &&
+            hipFuncSetAttribute(reinterpret_cast<const void *>(k), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                (int)wbytes) != hipSuccess)
+            return fail(TNN_ERR_HIP, "cannot reserve %zu bytes of LDS", wbytes);
+        hipLaunchKernelGGL(k, dim3((unsigned)blocks), dim3(kFwdThreads), wbytes, s, (const vec8 *)wprep_bwd,
+                           (const T *)dLdy, (const T *)interm_fwd, (T *)interm_bwd, (T *)dLdx, n_mats, d->activation,
+                           d->output_activation, (long long)M);
+    } else {
+        hipLaunchKernelGGL((mlp_backward_kernel<T, W, false>), dim3((unsigned)blocks), dim3(kFwdThreads), 0, s,
+                           (const vec8 *)wprep_bwd, (const T *)dLdy, (const T *)interm_fwd, (T *)interm_bwd, (T *)dLdx,
+                           n_mats, d->activation, d->output_activation, (long long)M);
+    }
+    return check_launch("mlp_backward_kernel");
+}
+
+struct DwPlan {
+    long long rows_per_chunk;
+    long long n_chunks;
+    int partials_per_chunk;
+    size_t partial_bytes; // fp32 partial tiles
+    size_t delta_bytes;   // staging for the deltas when the caller does not want them
+};
+
+static DwPlan dw_plan(const tnn_mlp_desc *d, size_t M) {
+    DwPlan p;
+    const int W = d->width, n_mats = d->n_hidden_layers + 1;
+    long long target_chunks = 256;
+    long long rpc = ((long long)M + target_chunks - 1) / target_chunks;
+    rpc = (rpc + kDwSlab - 1) / kDwSlab * kDwSlab;
+    if (rpc < kDwSlab) rpc = kDwSlab;
+    p.rows_per_chunk = rpc;
+    p.n_chunks = M ? ((long long)M + rpc - 1) / rpc : 0;
+    p.partials_per_chunk = (W <= 32) ? 4 : 1;
+    p.partial_bytes = (size_t)p.n_chunks * p.partials_per_chunk * n_mats * W * W * sizeof(float);
+    p.delta_bytes = (size_t)n_mats * M * W * 2;
+    return p;
+}
+
+template <typename T, int W>
+static int launch_dw(const tnn_mlp_desc *d, const void *interm_bwd, const void *interm_fwd, void *dW, int dW_is_fp32,
+                     size_t M, float *partials, hipStream_t s) {
+    const int n_mats = d->n_hidden_layers + 1;
+    const DwPlan p = dw_plan(d, M);
+    hipLaunchKernelGGL((mlp_dw_partial_kernel<T, W>), dim3((unsigned)p.n_chunks, (unsigned)n_mats), dim3(kDwThreads), 0, s,
+                       (const T *)interm_bwd, (const T *)interm_fwd, partials, n_mats, (long long)M, p.rows_per_chunk);
+    int rc = check_launch("mlp_dw_partial_kernel");
+    if (rc) return rc;
+    const int n_elems = n_mats * W * W;
+    hipLaunchKernelGGL((dw_reduce_kernel<T>), dim3((n_elems + 255) / 256), dim3(256), 0, s, partials,
+                       (int)(p.n_chunks * p.partials_per_chunk), n_elems, dW_is_fp32 ? (T *)nullptr : (T *)dW,
+                       dW_is_fp32 ? (float *)dW : (float *)nullptr);
+    return check_launch("dw_reduce_kernel");
+}
+
+#define TNN_DISPATCH_TW(desc, CALL)                                                          \
+    do {                                                                                     \
+        if ((desc)->dtype == TNN_BF16) {                                                     \
+            switch ((desc)->width) {                                                         \
+            case 16: { typedef bf16_t T_; constexpr int W_ = 16; CALL; } break;              \
+            case 32: { typedef bf16_t T_; constexpr int W_ = 32; CALL; } break;              \
+            case 64: { typedef bf16_t T_; constexpr int W_ = 64; CALL; } break;              \
+            default: { typedef bf16_t T_; constexpr int W_ = 128; CALL; } break;             \
+            }                                                                                \
+        } else {                                                                             \
+            switch ((desc)->width) {                                                         \
+            case 16: { typedef fp16_t T_; constexpr int W_ = 16; CALL; } break;              \
+            case 32: { typedef fp16_t T_; constexpr int W_ = 32; CALL; } break;              \
+            case 64: { typedef fp16_t T_; constexpr int W_ = 64; CALL; } break;              \
+            default: { typedef fp16_t T_; constexpr int W_ = 128; CALL; } break;             \
+            }                                                                                \
+        }                                                                                    \
+    } while (0)
+
+static int check_batch(size_t M) {
+    // include/network/SwiftNetMLP.h:293-300: the batch must be a multiple of 8
+    if (M == 0 || (M % 8) != 0) return fail(TNN_ERR_INVALID_ARGUMENT, "batch size %zu is not a positive multiple of 8", M);
+    return TNN_OK;
+}
+
+} // namespace tnn
+
+using namespace tnn;
+
+TNN_API size_t tnn_mlp_prepared_bytes(const tnn_mlp_desc *desc) {
+    if (check_mlp_desc(desc)) return 0;
+    return prepared_elems(desc) * 2;
+}
+
+TNN_API int tnn_mlp_prepare_weights(const tnn_mlp_desc *desc, const void *d_packed, int src_is_fp32, void *d_prepared_fwd,
+                                    void *d_prepared_bwd, tnn_stream_t stream) {
+    int rc = check_mlp_desc(desc);
+    if (rc) return rc;
+    if (!d_packed) return fail(TNN_ERR_INVALID_ARGUMENT, "d_packed is NULL");
+    const int n_mats = desc->n_hidden_layers + 1;
+    const int total = (int)prepared_elems(desc);
+    const int blocks = (total + 255) / 256;
+    hipStream_t s = as_stream(stream);
+    if (desc->dtype == TNN_BF16) {
+        if (src_is_fp32)
+            hipLaunchKernelGGL((prepare_weights_kernel<bf16_t, float>), dim3(blocks), dim3(256), 0, s, (const float *)d_packed,
+                               (bf16_t *)d_prepared_fwd, (bf16_t *)d_prepared_bwd, desc->width, n_mats);
+        else
+            hipLaunchKernelGGL((prepare_weights_kernel<bf16_t, bf16_t>), dim3(blocks), dim3(256), 0, s,
+                               (const bf16_t *)d_packed, (bf16_t *)d_prepared_fwd, (bf16_t *)d_prepared_bwd, desc->width,
+                               n_mats);
+    } else {
+        if (src_is_fp32)
+            hipLaunchKernelGGL((prepare_weights_kernel<fp16_t, float>), dim3(blocks), dim3(256), 0, s, (const float *)d_packed,
+                               (fp16_t *)d_prepared_fwd, (fp16_t *)d_prepared_bwd, desc->width, n_mats);
+        else
+            hipLaunchKernelGGL((prepare_weights_kernel<fp16_t, fp16_t>), dim3(blocks), dim3(256), 0, s,
+                               (const fp16_t *)d_packed, (fp16_t *)d_prepared_fwd, (fp16_t *)d_prepared_bwd, desc->width,
+                               n_mats);
+    }
+    return check_launch("prepare_weights_kernel");
+}
+
+TNN_API int tnn_mlp_inference(const tnn_mlp_desc *desc, const void *d_prepared_fwd, const void *d_x, void *d_y, size_t M,
+                              tnn_stream_t stream) {
+    int rc = check_mlp_desc(desc);
+    if (rc) return rc;
+    if ((rc = check_batch(M))) return rc;
+    if (!d_prepared_fwd || !d_x || !d_y) return fail(TNN_ERR_INVALID_ARGUMENT, "NULL pointer argument");
+    TNN_DISPATCH_TW(desc, rc = (launch_forward<T_, W_, false>(desc, d_prepared_fwd, d_x, d_y, M, as_stream(stream))));
+    return rc;
+}
+
+TNN_API int tnn_mlp_forward(const tnn_mlp_desc *desc, const void *d_prepared_fwd, const void *d_x, void *d_interm_fwd,
+                            size_t M, tnn_stream_t stream) {
+    int rc = check_mlp_desc(desc);
+    if (rc) return rc;
+    if ((rc = check_batch(M))) return rc;
+    if (!d_prepared_fwd || !d_x || !d_interm_fwd) return fail(TNN_ERR_INVALID_ARGUMENT, "NULL pointer argument");
+    TNN_DISPATCH_TW(desc, rc = (launch_forward<T_, W_, true>(desc, d_prepared_fwd, d_x, d_interm_fwd, M, as_stream(stream))));
+    return rc;
+}
+
+TNN_API size_t tnn_mlp_backward_workspace_bytes(const tnn_mlp_desc *desc, size_t M) {
+    if (check_mlp_desc(desc)) return 0;
+    const DwPlan p = dw_plan(desc, M);
+    return ((p.partial_bytes + 255) & ~(size_t)255) + p.delta_bytes + 512;
+}
+
+TNN_API int tnn_mlp_backward(const tnn_mlp_desc *desc, const void *d_prepared_bwd, const void *d_dLdy,
+                             const void *d_interm_fwd, void *d_interm_bwd, void *d_dW, int dW_is_fp32, void *d_dLdx,
+                             size_t M, void *d_workspace, size_t workspace_bytes, tnn_stream_t stream) {
+    int rc = check_mlp_desc(desc);
+    if (rc) return rc;
+    if ((rc = check_batch(M))) return rc;
+    if (!d_prepared_bwd || !d_dLdy || !d_interm_fwd || !d_dW) return fail(TNN_ERR_INVALID_ARGUMENT, "NULL pointer argument");
+    const DwPlan p = dw_plan(desc, M);
+    const size_t partial_rounded = (p.partial_bytes + 255) & ~(size_t)255;
+    const size_t need = partial_rounded + (d_interm_bwd ? 0 : p.delta_bytes) + 512;
+    if (!d_workspace || workspace_bytes < need)
+        return fail(TNN_ERR_WORKSPACE, "workspace of %zu bytes given, %zu needed", workspace_bytes, need);
+    // 256-byte aligned partial tiles first, delta staging after them
+    uintptr_t base = (reinterpret_cast<uintptr_t>(d_workspace) + 255) & ~(uintptr_t)255;
+    float *partials = reinterpret_cast<float *>(base);
+    void *deltas = d_interm_bwd ? d_interm_bwd : reinterpret_cast<void *>(base + partial_rounded);
+    hipStream_t s = as_stream(stream);
+    TNN_DISPATCH_TW(desc, rc = (launch_backward<T_, W_>(desc, d_prepared_bwd, d_dLdy, d_interm_fwd, deltas, d_dLdx, M, s)));
+    if (rc) return rc;
+    TNN_DISPATCH_TW(desc, rc = (launch_dw<T_, W_>(desc, deltas, d_interm_fwd, d_dW, dW_is_fp32, M, partials, s)));
+    return rc;
+}

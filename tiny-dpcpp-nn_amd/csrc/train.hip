@@ -1,0 +1,80 @@
+// One training step of the fused MLP against an L2 loss: forward, loss + gradient, backward with
+// weight gradients (include/trainer.h:23-46 with include/losses/l2.h:19-40 in between).
+#include "tnn_internal.h"
+
+namespace tnn {
+
+// loss value summed per workgroup, one atomic per workgroup; gradient rounded to T as in l2.h:24
+template <typename T>
+__global__ void __launch_bounds__(256)
+    l2_loss_sum_kernel(const T *__restrict__ pred, const float *__restrict__ target, size_t n, float inv_n, float loss_scale,
+                       float *__restrict__ loss_sum, T *__restrict__ grads) {
+    __shared__ float red[4];
+    float local = 0.0f;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
+        const float diff = (float)pred[i] - target[i];
+        local += diff * diff * inv_n;
+        grads[i] = (T)(loss_scale * 2 * diff * inv_n);
+    }
+    if (loss_sum) {
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) local += __shfl_down(local, off, 64);
+        if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = local;
+        __syncthreads();
+        if (threadIdx.x == 0) unsafeAtomicAdd(loss_sum, red[0] + red[1] + red[2] + red[3]);
+    }
+}
+
+__global__ void zero_scalar_kernel(float *p) { *p = 0.0f; }
+
+static size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
+
+} // namespace tnn
+
+using namespace tnn;
+
+TNN_API size_t tnn_mlp_train_step_workspace_bytes(const tnn_mlp_desc *desc, size_t M) {
+    if (check_mlp_desc(desc)) return 0;
+    const size_t mat = M * desc->width * 2;
+    return align256((size_t)(desc->n_hidden_layers + 2) * mat) + align256(mat) + tnn_mlp_backward_workspace_bytes(desc, M) + 512;
+}
+
+TNN_API int tnn_mlp_train_step_l2(const tnn_mlp_desc *desc, const void *d_prepared_fwd, const void *d_prepared_bwd,
+                                  const void *d_x, const float *d_targets, float loss_scale, void *d_y, float *d_loss_sum,
+                                  void *d_dW, int dW_is_fp32, void *d_dLdx, size_t M, void *d_workspace,
+                                  size_t workspace_bytes, tnn_stream_t stream) {
+    int rc = check_mlp_desc(desc);
+    if (rc) return rc;
+    if (!d_prepared_fwd || !d_prepared_bwd || !d_x || !d_targets || !d_dW) return fail(TNN_ERR_INVALID_ARGUMENT, "NULL pointer argument");
+    if (loss_scale == 0.0f) return fail(TNN_ERR_INVALID_ARGUMENT, "loss_scale must not be 0");
+    const size_t need = tnn_mlp_train_step_workspace_bytes(desc, M);
+    if (!d_workspace || workspace_bytes < need)
+        return fail(TNN_ERR_WORKSPACE, "workspace of %zu bytes given, %zu needed", workspace_bytes, need);
+    hipStream_t s = as_stream(stream);
+    const int W = desc->width, n_mats = desc->n_hidden_layers + 1;
+    const size_t mat = M * W * 2;
+    uintptr_t base = align256(reinterpret_cast<uintptr_t>(d_workspace));
+    void *interm_fwd = reinterpret_cast<void *>(base);
+    base += align256((size_t)(n_mats + 1) * mat);
+    void *dLdy = reinterpret_cast<void *>(base);
+    base += align256(mat);
+    void *bwd_ws = reinterpret_cast<void *>(base);
+    const size_t bwd_ws_bytes = workspace_bytes - (base - reinterpret_cast<uintptr_t>(d_workspace));
+
+    if ((rc = tnn_mlp_forward(desc, d_prepared_fwd, d_x, interm_fwd, M, stream))) return rc;
+    const void *y = static_cast<const char *>(interm_fwd) + (size_t)n_mats * mat;
+    if (d_y && hipMemcpyAsync(d_y, y, mat, hipMemcpyDeviceToDevice, s) != hipSuccess) return fail(TNN_ERR_HIP, "copy of the network output failed");
+    const size_t n = M * W;
+    if (d_loss_sum) hipLaunchKernelGGL(zero_scalar_kernel, dim3(1), dim3(1), 0, s, d_loss_sum);
+    size_t blocks = (n + 256 * 8 - 1) / (256 * 8);
+    if (blocks > 2048) blocks = 2048;
+    const float inv_n = 1.0f / (float)n;
+    if (desc->dtype == TNN_BF16)
+        hipLaunchKernelGGL((l2_loss_sum_kernel<bf16_t>), dim3((unsigned)blocks), dim3(256), 0, s, (const bf16_t *)y, d_targets, n, inv_n,
+                           loss_scale, d_loss_sum, (bf16_t *)dLdy);
+    else
+        hipLaunchKernelGGL((l2_loss_sum_kernel<fp16_t>), dim3((unsigned)blocks), dim3(256), 0, s, (const fp16_t *)y, d_targets, n, inv_n,
+                           loss_scale, d_loss_sum, (fp16_t *)dLdy);
+    if ((rc = check_launch("l2_loss_sum_kernel"))) return rc;
+    return tnn_mlp_backward(desc, d_prepared_bwd, dLdy, interm_fwd, nullptr, d_dW, dW_is_fp32, d_dLdx, M, bwd_ws, bwd_ws_bytes, stream);
+}

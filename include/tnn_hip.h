@@ -123,8 +123,8 @@ int tnn_mlp_inference(const tnn_mlp_desc *desc, const void *d_prepared_fwd, cons
 int tnn_mlp_forward(const tnn_mlp_desc *desc, const void *d_prepared_fwd, const void *d_x, void *d_interm_fwd, size_t M,
                     tnn_stream_t stream);
 
-/* Workspace bytes tnn_mlp_backward / tnn_mlp_train_step_l2 need for their per-workgroup fp32
- * partial weight gradients. */
+/* Workspace bytes tnn_mlp_backward needs (fp32 partial weight gradients, and staging for the deltas
+ * when d_interm_bwd is NULL). */
 size_t tnn_mlp_backward_workspace_bytes(const tnn_mlp_desc *desc, size_t M);
 
 /* EsimdKernels::backward_impl (include/network/kernel_esimd.h:160-240: fused delta propagation
@@ -132,7 +132,7 @@ size_t tnn_mlp_backward_workspace_bytes(const tnn_mlp_desc *desc, size_t M);
  * (include/network/SwiftNetMLP.h:199-248).
  *   d_dLdy: M x W T. d_interm_fwd: as written by tnn_mlp_forward.
  *   d_interm_bwd: (n_hidden_layers + 1) matrices M x W, [l] = delta_l; may be NULL (then the deltas
- *                 never leave the chip).
+ *                 are staged in the workspace).
  *   d_dW: (n_hidden_layers + 1) matrices [n=out][k=in] row-major T, unpacked (the gemm_batch output).
  *         If dW_is_fp32 != 0 the same layout is written as fp32 without the final rounding.
  *   d_dLdx: M x W T or NULL (kernel_esimd.h:217-226). */
@@ -145,9 +145,13 @@ int tnn_mlp_backward(const tnn_mlp_desc *desc, const void *d_prepared_bwd, const
 int tnn_l2_loss(int dtype, const void *d_predictions, const float *d_targets, size_t n_elements, float loss_scale,
                 float *d_values, void *d_grads, tnn_stream_t stream);
 
-/* One fused training step of the MLP: forward, L2 loss against fp32 targets, backward with weight
- * gradients, with no activation or delta written to device memory. Equivalent to
- * Trainer::training_step (include/trainer.h:23-46) with L2Loss::evaluate in between.
+/* Workspace bytes for tnn_mlp_train_step_l2. */
+size_t tnn_mlp_train_step_workspace_bytes(const tnn_mlp_desc *desc, size_t M);
+
+/* One training step of the MLP in a single call: forward, L2 loss against fp32 targets, backward
+ * with weight gradients. Equivalent to Trainer::training_step (include/trainer.h:23-46) with
+ * L2Loss::evaluate (include/losses/loss.h:19-25) between its forward and backward pass; the
+ * intermediate activations and deltas live in the workspace instead of caller-visible matrices.
  *   d_y: M x W network output (T) or NULL. d_loss_sum: one fp32 that receives sum_i value_i
  *   (the mean squared error), or NULL. d_dW / dW_is_fp32 / d_dLdx as in tnn_mlp_backward.
  *   N of the loss = M * W (all padded columns count, as in the reference). */

@@ -1,0 +1,57 @@
+"""CPU-side checks of the C-ABI library: it loads, exports every symbol include/tnn_hip.h declares,
+and its pure host entry points (descriptor validation, size queries) behave. No kernel is launched."""
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    txt = open(os.path.join(ROOT, "include", "tnn_hip.h")).read()
+    txt = re.sub(r"/\*.*?\*/", "", txt, flags=re.S)
+    return sorted(set(re.findall(r"\b(tnn_[a-z0-9_]+)\s*\(", txt)))
+
+
+@pytest.fixture(scope="module")
+def lib():
+    from tiny_dpcpp_nn import _lib
+    return _lib.load()
+
+
+def test_exports_every_declared_symbol(lib):
+    from tiny_dpcpp_nn import _lib
+    names = declared_symbols()
+    assert len(names) >= 20
+    for n in names:
+        assert hasattr(lib, n), f"{n} is declared in include/tnn_hip.h but not exported"
+        assert n in _lib.SIGNATURES, f"{n} has no ctypes prototype"
+    assert lib.tnn_abi_version() == 1
+
+
+def test_descriptor_validation_is_host_only(lib):
+    from tiny_dpcpp_nn import _lib
+    good = _lib.MlpDesc(_lib.TNN_BF16, 64, 4, _lib.ACT_RELU, _lib.ACT_NONE)
+    # (4+1) matrices * 2 tiles * 4 k-blocks * 512 elements * 2 bytes
+    assert lib.tnn_mlp_prepared_bytes(ctypes.byref(good)) == 5 * 2 * 4 * 512 * 2
+    assert lib.tnn_mlp_prepared_bytes(ctypes.byref(_lib.MlpDesc(_lib.TNN_FP16, 16, 2, 0, 8))) == 3 * 1 * 1 * 512 * 2
+    for bad in (_lib.MlpDesc(_lib.TNN_BF16, 48, 4, 0, 8), _lib.MlpDesc(_lib.TNN_BF16, 64, 0, 0, 8), _lib.MlpDesc(_lib.TNN_FP32, 64, 4, 0, 8),
+                _lib.MlpDesc(_lib.TNN_BF16, 64, 4, _lib.ACT_TANH, 8)):
+        assert lib.tnn_mlp_prepared_bytes(ctypes.byref(bad)) == 0
+        assert lib.tnn_mlp_backward_workspace_bytes(ctypes.byref(bad), 1024) == 0
+    assert lib.tnn_mlp_backward_workspace_bytes(ctypes.byref(good), 1 << 18) > 0
+    assert lib.tnn_mlp_train_step_workspace_bytes(ctypes.byref(good), 1 << 18) > lib.tnn_mlp_backward_workspace_bytes(ctypes.byref(good), 1 << 18)
+
+
+def test_grid_descriptor_host_side(lib):
+    from tiny_dpcpp_nn import _lib
+    d = _lib.GridDesc()
+    assert lib.tnn_grid_desc_init(ctypes.byref(d), 2, 16, 2, 19, 16, 1.5, 0, 1, 1, _lib.TNN_FP16) == 0
+    assert d.offsets[16] == 3829192 and lib.tnn_grid_n_params(ctypes.byref(d)) == 7658384
+    assert lib.tnn_grid_desc_init(ctypes.byref(d), 3, 16, 2, 22, 16, 1.447, 0, 1, 1, _lib.TNN_FP16) == 0
+    assert d.offsets[16] == 42519264
+    assert lib.tnn_grid_desc_init(ctypes.byref(d), 3, 200, 2, 22, 16, 1.447, 0, 1, 1, _lib.TNN_FP16) == _lib.TNN_ERR_INVALID_ARGUMENT
+    assert b"MAX_N_LEVELS" in lib.tnn_last_error()
+    assert lib.tnn_grid_desc_init(ctypes.byref(d), 5, 16, 2, 22, 16, 1.447, 0, 1, 1, _lib.TNN_FP16) == _lib.TNN_ERR_UNSUPPORTED

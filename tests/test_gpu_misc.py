@@ -1,0 +1,55 @@
+"""L2 loss and Adam kernels against the oracle."""
+import numpy as np
+import pytest
+import torch
+
+from tolerances import BF16, FP16, FP32
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("dtype,tdt", [(BF16, torch.bfloat16), (FP16, torch.float16)])
+def test_l2_loss(tnn, oracle, dtype, tdt):
+    rng = np.random.default_rng(0)
+    M, W = 1024, 64
+    pred = oracle.round(rng.standard_normal((M, W)), dtype)
+    targ = rng.uniform(0, 1, (M, W)).astype(np.float32)
+    for ls in (1.0, 128.0, 10.0):
+        values, grads = tnn.l2_loss(dtype, torch.from_numpy(pred).to(tnn.dev).to(tdt), torch.from_numpy(targ).to(tnn.dev), ls)
+        rv, rg = oracle.l2_loss(dtype, pred, targ, ls)
+        assert np.allclose(values.cpu().numpy(), rv, rtol=1e-6, atol=0)
+        assert np.array_equal(tnn.host(grads), rg)  # same fp32 expression, same rounding: bit-exact
+    # closed form of test/doctest_losses.cpp:46-51
+    p = torch.full((8, 16), 0.5, device=tnn.dev).to(tdt)
+    t = torch.full((8, 16), 0.125, device=tnn.dev)
+    values, grads = tnn.l2_loss(dtype, p, t, 4.0)
+    assert np.allclose(values.cpu().numpy(), 0.375 ** 2 / 128)
+    assert np.allclose(tnn.host(grads), 4.0 * 2 * 0.375 / 128, rtol=4e-3)
+
+
+def test_adam(tnn, oracle):
+    rng = np.random.default_rng(1)
+    n = 20480
+    p0 = rng.standard_normal(n).astype(np.float32) * 0.1
+    p = torch.from_numpy(p0.copy()).to(tnn.dev)
+    m = torch.zeros_like(p)
+    v = torch.zeros_like(p)
+    rp, rm, rv = p0.copy(), np.zeros(n, np.float32), np.zeros(n, np.float32)
+    tp = torch.nn.Parameter(torch.from_numpy(p0.copy()))
+    opt = torch.optim.Adam([tp], lr=1e-3, betas=(0.9, 0.99), eps=1e-15)
+    pT = torch.empty(n, dtype=torch.float16, device=tnn.dev)
+    for step in range(1, 5):
+        g = (rng.standard_normal(n) * 128).astype(np.float32)
+        gs = 1.0 / 128
+        tnn.adam_step(p, m, v, torch.from_numpy(g).to(tnn.dev), FP32, gs, step, 1e-3, 0.9, 0.99, 1e-15, pT, FP16)
+        rp, rm, rv = oracle.adam_step(rp, rm, rv, g * np.float32(gs), step, 1e-3, 0.9, 0.99, 1e-15)
+        tp.grad = torch.from_numpy(g * np.float32(gs))
+        opt.step()
+        assert np.allclose(tnn.host(p), rp, rtol=1e-6, atol=1e-7)
+        assert np.allclose(tnn.host(p), tp.detach().numpy(), rtol=1e-6, atol=1e-7)
+    assert np.array_equal(tnn.host(pT), oracle.round(tnn.host(p), FP16))
+    # half-precision gradients
+    g16 = oracle.round(rng.standard_normal(n), BF16)
+    tnn.adam_step(p, m, v, torch.from_numpy(g16).to(tnn.dev).to(torch.bfloat16), BF16, 1.0, 5, 1e-3, 0.9, 0.99, 1e-15)
+    rp, rm, rv = oracle.adam_step(rp, rm, rv, g16, 5, 1e-3, 0.9, 0.99, 1e-15)
+    assert np.allclose(tnn.host(p), rp, rtol=1e-6, atol=1e-7)

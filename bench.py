@@ -1,0 +1,276 @@
+#!/usr/bin/env python3
+"""Benchmark of the hot path on one MI355X.
+
+Default workload (BASELINE config 2, the one the metric is quoted on): one training step of the
+width-64, 4-hidden-layer bf16 fused MLP at batch 2^18 -- forward, L2 loss against U[0,1) targets,
+backward with weight gradients, Adam (lr 1e-3, betas 0.9/0.99, eps 1e-15) on fp32 master weights and
+re-staging of the updated weights for the next step. Inputs are resident in HBM before the timed
+region. Prints ONE JSON line.
+
+Other workloads (reported as extra lines only when asked for with --workload):
+  infer  BASELINE config 1 shape at batch 2^18: fused inference
+  grid   BASELINE config 5 encoding: 3-D hash grid forward, 2^21 points
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(ROOT, "tiny-dpcpp-nn_amd"))
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+PEAK_MFMA_BF16 = 2500.0  # TFLOP/s, dense
+PEAK_HBM = 8000.0  # GB/s
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default="train", choices=["train", "infer", "grid"])
+    ap.add_argument("--batch-log2", type=int, default=None)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    return ap.parse_args()
+
+
+def cpu_baseline_train(oracle, W, n_mats, budget_s=12.0):
+    """The oracle's training step (rounding-point restatement) timed on the host cores on a bounded sample."""
+    import numpy as np
+    from tolerances import BF16
+
+    rng = np.random.default_rng(0)
+    lim = np.sqrt(6.0 / (2 * W))
+    w = oracle.round(rng.uniform(-lim, lim, (n_mats, W, W)), BF16)
+    cores = oracle.num_threads()
+    M = 1 << 14
+    x = oracle.round(rng.uniform(-1, 1, (M, W)), BF16)
+    tg = rng.uniform(0, 1, (M, W)).astype(np.float32)
+
+    def step():
+        interm = oracle.mlp_forward_T(BF16, W, n_mats, "relu", "none", w, x)
+        _, g = oracle.l2_loss(BF16, interm[-1], tg, 1.0)
+        oracle.mlp_backward_T(BF16, W, n_mats, "relu", "none", w, interm, g, want_dx=False, round_dw=False)
+
+    step()
+    t0 = time.perf_counter()
+    n = 0
+    while time.perf_counter() - t0 < budget_s:
+        step()
+        n += 1
+    dt = time.perf_counter() - t0
+    return {"value": M * n / dt, "unit": "samples/s", "cores": cores, "kind": "port",
+            "sample": f"{n} training steps (forward, L2, backward with dW) of {M} rows each, w64 / 4 hidden layers, bf16 rounding points, OpenMP over rows"}
+
+
+def cpu_baseline_infer(oracle, W, n_mats, budget_s=12.0):
+    import numpy as np
+    from tolerances import BF16
+
+    rng = np.random.default_rng(0)
+    lim = np.sqrt(6.0 / (2 * W))
+    w = oracle.round(rng.uniform(-lim, lim, (n_mats, W, W)), BF16)
+    M = 1 << 15
+    x = oracle.round(rng.uniform(-1, 1, (M, W)), BF16)
+    oracle.mlp_forward_T(BF16, W, n_mats, "relu", "none", w, x, store_interm=False)
+    t0 = time.perf_counter()
+    n = 0
+    while time.perf_counter() - t0 < budget_s:
+        oracle.mlp_forward_T(BF16, W, n_mats, "relu", "none", w, x, store_interm=False)
+        n += 1
+    dt = time.perf_counter() - t0
+    return {"value": M * n / dt, "unit": "samples/s", "cores": oracle.num_threads(), "kind": "port",
+            "sample": f"{n} inference passes of {M} rows, w64 / 4 hidden layers, bf16 rounding points, OpenMP over rows"}
+
+
+def cpu_baseline_grid(oracle, cfg, budget_s=12.0):
+    import numpy as np
+    from tolerances import FP16
+
+    rng = np.random.default_rng(0)
+    off, _, _ = oracle.grid_offsets(cfg["n_dims"], cfg["n_levels"], cfg["log2_hashmap_size"], cfg["base_resolution"], cfg["per_level_scale"])
+    n = int(off[-1]) * cfg["n_features_per_level"]
+    table = oracle.round(rng.uniform(-1e-4, 1e-4, n), FP16)
+    M = 1 << 16
+    x = rng.uniform(0, 1, (M, cfg["n_dims"])).astype(np.float32)
+    oracle.grid_forward(cfg, table, x, 32)
+    t0 = time.perf_counter()
+    k = 0
+    while time.perf_counter() - t0 < budget_s:
+        oracle.grid_forward(cfg, table, x, 32)
+        k += 1
+    dt = time.perf_counter() - t0
+    return {"value": M * k / dt, "unit": "points/s", "cores": oracle.num_threads(), "kind": "port",
+            "sample": f"{k} forward passes of {M} points through the full 162 MiB table, OpenMP over points"}
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (every row is independent; see DESIGN.md "
+              "for how it would shard). Run with --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+
+    import gpu_harness
+    import oracle_bindings
+    from gpu_harness import ptr
+    from tiny_dpcpp_nn import _lib
+    from tolerances import BF16, FP16, FP32
+
+    t = gpu_harness.Harness()
+    lib = t.lib
+    oracle = None
+    if not args.no_cpu_baseline:
+        oracle = oracle_bindings.Oracle(os.path.join(ROOT, "oracle", "libtnn_oracle.so"))
+
+    K, Wm = args.steps, args.warmup
+    ev = lambda: torch.cuda.Event(enable_timing=True)
+    out = {}
+
+    if args.workload in ("train", "infer"):
+        W, n_hidden = 64, 4
+        n_mats = n_hidden + 1
+        M = 1 << (args.batch_log2 or 18)
+        desc = t.mlp_desc(BF16, W, n_hidden, "relu", "none")
+        rng = np.random.default_rng(42)
+        lim = np.sqrt(6.0 / (2 * W))
+        w = rng.uniform(-lim, lim, (n_mats, W, W)).astype(np.float32)
+        gen = torch.Generator(device=t.dev).manual_seed(1234)
+        x = (torch.rand((M, W), device=t.dev, generator=gen) * 2 - 1).to(torch.bfloat16)
+        # fp32 master weights in the packed parameter layout, as the reference's Python module keeps them
+        master = t.pack(FP32, W, n_mats, torch.from_numpy(w.reshape(-1)).to(t.dev))
+        pf, pb = t.prepare_packed(desc, master, src_is_fp32=True)
+
+    if args.workload == "train":
+        targets = torch.rand((M, W), device=t.dev, generator=gen)
+        ws_bytes = lib.tnn_mlp_train_step_workspace_bytes(ctypes.byref(desc), M)
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=t.dev)
+        dW = torch.empty((n_mats, W, W), dtype=torch.float32, device=t.dev)
+        dWp = torch.empty_like(dW)
+        loss = torch.zeros(1, device=t.dev)
+        m = torch.zeros_like(master)
+        v = torch.zeros_like(master)
+        s = t.stream()
+        d = ctypes.byref(desc)
+        ks, ke = [ev() for _ in range(K)], [ev() for _ in range(K)]
+
+        def step(i, timed=-1):
+            if timed >= 0:
+                ks[timed].record()
+            rc = lib.tnn_mlp_train_step_l2(d, ptr(pf), ptr(pb), ptr(x), ptr(targets), 1.0, None, ptr(loss), ptr(dW), 1, None, M,
+                                           ptr(ws), ws_bytes, s)
+            if timed >= 0:
+                ke[timed].record()
+            rc |= lib.tnn_pack_and_transpose(FP32, W, n_mats, ptr(dW), ptr(dWp), s)
+            rc |= lib.tnn_adam_step(ptr(master), ptr(m), ptr(v), ptr(dWp), FP32, 1.0, master.numel(), i + 1, 1e-3, 0.9, 0.99, 1e-15, None, BF16, s)
+            rc |= lib.tnn_mlp_prepare_weights(d, ptr(master), 1, ptr(pf), ptr(pb), s)
+            if rc:
+                raise RuntimeError(lib.tnn_last_error())
+
+        for i in range(Wm):
+            step(i)
+        torch.cuda.synchronize()
+        loss0 = float(loss.item())
+        e0, e1 = ev(), ev()
+        t0 = time.perf_counter()
+        e0.record()
+        for i in range(K):
+            step(Wm + i, timed=i)
+        e1.record()
+        torch.cuda.synchronize()
+        wall = time.perf_counter() - t0
+        ms = e0.elapsed_time(e1) / K
+        kern_ms = sum(a.elapsed_time(b) for a, b in zip(ks, ke)) / K
+        flops = 3 * 2 * M * W * W * n_mats  # reference convention: forward + backward-data + dW
+        out = {
+            "metric": "fused-MLP train & infer samples/s (w64, batch 2^18); % bf16 MFMA peak",
+            "value": M / (ms * 1e-3), "unit": "samples/s", "n_gpus": 1, "steps": K, "warmup": Wm, "ms_per_step": ms,
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+            "config": {"workload": f"training step: w64, 4 hidden layers (5 matmuls), ReLU/linear, bf16, batch 2^{int(np.log2(M))}, "
+                                   "L2 loss, Adam on fp32 masters (BASELINE config 2)", "batch": M},
+            "roofline": {"bound": "mfma", "achieved": flops / (kern_ms * 1e-3) / 1e12, "peak": PEAK_MFMA_BF16, "unit": "TFLOP/s",
+                         "frac": flops / (kern_ms * 1e-3) / 1e12 / PEAK_MFMA_BF16, "traffic": None,
+                         "kernel": "tnn_mlp_train_step_l2 (forward + loss + backward + dW)", "kernel_ms": kern_ms,
+                         "algorithmic_flops_per_launch": flops},
+            "mfma_frac_whole_step": flops / (ms * 1e-3) / 1e12 / PEAK_MFMA_BF16,
+            "wall_ms_per_step": wall / K * 1e3,
+            "loss_first": loss0, "loss_last": float(loss.item()),
+        }
+        if oracle is not None:
+            out["cpu_baseline"] = cpu_baseline_train(oracle, W, n_mats)
+
+    elif args.workload == "infer":
+        y = torch.empty_like(x)
+        s = t.stream()
+        d = ctypes.byref(desc)
+        for _ in range(Wm):
+            lib.tnn_mlp_inference(d, ptr(pf), ptr(x), ptr(y), M, s)
+        torch.cuda.synchronize()
+        e0, e1 = ev(), ev()
+        e0.record()
+        for _ in range(K):
+            lib.tnn_mlp_inference(d, ptr(pf), ptr(x), ptr(y), M, s)
+        e1.record()
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1) / K
+        flops = 2 * M * W * W * n_mats
+        bytes_ = 2 * M * W * 2 + n_mats * W * W * 2
+        out = {
+            "metric": "fused-MLP train & infer samples/s (w64, batch 2^18); % bf16 MFMA peak",
+            "value": M / (ms * 1e-3), "unit": "samples/s", "n_gpus": 1, "steps": K, "warmup": Wm, "ms_per_step": ms,
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+            "config": {"workload": f"inference: w64, 4 hidden layers (5 matmuls), ReLU/linear, bf16, batch 2^{int(np.log2(M))} (BASELINE config 1 shape)",
+                       "batch": M},
+            "roofline": {"bound": "hbm", "achieved": bytes_ / (ms * 1e-3) / 1e9, "peak": PEAK_HBM, "unit": "GB/s",
+                         "frac": bytes_ / (ms * 1e-3) / 1e9 / PEAK_HBM, "traffic": None, "kernel": "mlp_forward_kernel (inference)",
+                         "kernel_ms": ms, "algorithmic_bytes_per_launch": bytes_},
+            "mfma_frac": flops / (ms * 1e-3) / 1e12 / PEAK_MFMA_BF16,
+        }
+        if oracle is not None:
+            out["cpu_baseline"] = cpu_baseline_infer(oracle, W, n_mats)
+
+    else:
+        cfg = dict(n_dims=3, n_levels=16, n_features_per_level=2, log2_hashmap_size=22, base_resolution=16, per_level_scale=1.447)
+        M = 1 << (args.batch_log2 or 21)
+        gd = t.grid_desc(cfg, FP16)
+        n = t.grid_n_params(gd)
+        gen = torch.Generator(device=t.dev).manual_seed(7)
+        table = (torch.rand(n, device=t.dev, generator=gen) * 2e-4 - 1e-4).to(torch.float16)
+        x = torch.rand((M, 3), device=t.dev, generator=gen)
+        o = torch.empty((M, 32), dtype=torch.float16, device=t.dev)
+        s = t.stream()
+        K = min(K, 50)
+        for _ in range(min(Wm, 5)):
+            lib.tnn_grid_forward(ctypes.byref(gd), ptr(x), ptr(table), ptr(o), FP16, 32, M, s)
+        torch.cuda.synchronize()
+        e0, e1 = ev(), ev()
+        e0.record()
+        for _ in range(K):
+            lib.tnn_grid_forward(ctypes.byref(gd), ptr(x), ptr(table), ptr(o), FP16, 32, M, s)
+        e1.record()
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1) / K
+        bpp = 12 + 16 * 8 * 4 + 32 * 2
+        out = {
+            "metric": "hash-grid forward points/s (3-D, 16x2, log2 22, fp16 table, batch 2^21); % HBM peak",
+            "value": M / (ms * 1e-3), "unit": "points/s", "n_gpus": 1, "steps": K, "warmup": min(Wm, 5), "ms_per_step": ms,
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+            "config": {"workload": f"3-D hash-grid encoding forward, 2^{int(np.log2(M))} points (BASELINE config 5 encoding)", "batch": M},
+            "roofline": {"bound": "hbm", "achieved": bpp * M / (ms * 1e-3) / 1e9, "peak": PEAK_HBM, "unit": "GB/s",
+                         "frac": bpp * M / (ms * 1e-3) / 1e9 / PEAK_HBM, "traffic": None, "kernel": "grid_forward_kernel",
+                         "kernel_ms": ms, "algorithmic_bytes_per_launch": bpp * M},
+        }
+        if oracle is not None:
+            out["cpu_baseline"] = cpu_baseline_grid(oracle, cfg)
+
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -90,7 +90,7 @@ __global__ void l2_loss_kernel(const T *__restrict__ pred, const float *__restri
     if (i >= n) return;
     const float diff = (float)pred[i] - target[i];
     if (values) values[i] = diff * diff * inv_n;
-    grads[i] = (T)(loss_scale * 2 * diff * inv_n);
+    grads[i] = (T)as_fp32(loss_scale * 2 * diff * inv_n);
 }
 
 template <typename G, typename P>

@@ -57,6 +57,14 @@ template <> struct Storage<fp16_t> {
     }
 };
 
+// Pins a value in a VGPR as an fp32 number. The reference rounds an fp32 product to fp32 first and to the
+// 2-byte type afterwards; without this the compiler merges "multiply, then narrow" into one mixed-precision
+// instruction that rounds once, which differs on exact ties.
+__device__ __forceinline__ float as_fp32(float v) {
+    asm volatile("" : "+v"(v));
+    return v;
+}
+
 // Swaps bits 2 and 3 of a 5-bit index. Row i of a 32-row MFMA output tile is held by lane half
 // h = bit 2 in accumulator register 4*(i>>3) + (i&3); storing weight column (32a + swap23(i)) in
 // operand row i makes every lane end up with 8 consecutive features per 16-feature block, which is

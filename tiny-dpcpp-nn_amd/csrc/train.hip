@@ -14,7 +14,7 @@ __global__ void __launch_bounds__(256)
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
         const float diff = (float)pred[i] - target[i];
         local += diff * diff * inv_n;
-        grads[i] = (T)(loss_scale * 2 * diff * inv_n);
+        grads[i] = (T)as_fp32(loss_scale * 2 * diff * inv_n);
     }
     if (loss_sum) {
 #pragma unroll
@@ -29,12 +29,19 @@ __global__ void zero_scalar_kernel(float *p) { *p = 0.0f; }
 
 static size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 
+// mlp_train.hip
+int fused_train_step(const tnn_mlp_desc *d, const void *wf, const void *wb, const void *x, const float *targets, float loss_scale,
+                     void *y, float *loss_sum, void *dW, int dW_is_fp32, void *dx, size_t M, void *ws, size_t ws_bytes, hipStream_t s);
+size_t fused_train_workspace_bytes(const tnn_mlp_desc *d, size_t M);
+
 } // namespace tnn
 
 using namespace tnn;
 
 TNN_API size_t tnn_mlp_train_step_workspace_bytes(const tnn_mlp_desc *desc, size_t M) {
     if (check_mlp_desc(desc)) return 0;
+    const size_t fused = fused_train_workspace_bytes(desc, M);
+    if (fused) return fused;
     const size_t mat = M * desc->width * 2;
     return align256((size_t)(desc->n_hidden_layers + 2) * mat) + align256(mat) + tnn_mlp_backward_workspace_bytes(desc, M) + 512;
 }
@@ -51,6 +58,12 @@ TNN_API int tnn_mlp_train_step_l2(const tnn_mlp_desc *desc, const void *d_prepar
     if (!d_workspace || workspace_bytes < need)
         return fail(TNN_ERR_WORKSPACE, "workspace of %zu bytes given, %zu needed", workspace_bytes, need);
     hipStream_t s = as_stream(stream);
+    if (M == 0 || (M % 8) != 0) return fail(TNN_ERR_INVALID_ARGUMENT, "batch size %zu is not a positive multiple of 8", M);
+    // shapes with a fused kernel never touch device memory with activations or deltas
+    rc = fused_train_step(desc, d_prepared_fwd, d_prepared_bwd, d_x, d_targets, loss_scale, d_y, d_loss_sum, d_dW, dW_is_fp32, d_dLdx, M,
+                          d_workspace, workspace_bytes, s);
+    if (rc != TNN_ERR_UNSUPPORTED) return rc;
+    // wider / deeper networks: forward, loss and backward as separate kernels over workspace matrices
     const int W = desc->width, n_mats = desc->n_hidden_layers + 1;
     const size_t mat = M * W * 2;
     uintptr_t base = align256(reinterpret_cast<uintptr_t>(d_workspace));

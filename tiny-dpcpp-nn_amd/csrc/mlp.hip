@@ -13,6 +13,8 @@
 // the fp32 accumulator before rounding).
 #include "mlp_tile.h"
 
+#include <cstdlib>
+
 namespace tnn {
 
 // ------------------------------------------------------------------------------------------
@@ -55,16 +57,18 @@ __global__ void prepare_weights_kernel(const SRC *__restrict__ packed, T *__rest
 // Forward / inference
 // ------------------------------------------------------------------------------------------
 // out: STORE_INTERM ? (n_mats + 1) matrices M x W ([0] = copy of x) : one matrix M x W.
-template <typename T, int W, bool STORE_INTERM, bool W_IN_LDS>
-__global__ void __launch_bounds__(kFwdThreads)
+// ACT (hidden activation) is a compile-time constant so that the layer loop stays one basic block:
+// the fragments of the next matrix are requested from LDS before the current accumulators are
+// converted, and arrive while the conversion runs.
+template <typename T, int W, int ACT, bool STORE_INTERM, bool W_IN_LDS, int THREADS, bool PREFETCH>
+__global__ void __launch_bounds__(THREADS, (THREADS == 512 && W <= 64) ? 4 : 1)
     mlp_forward_kernel(const typename Storage<T>::vec8 *__restrict__ wprep, const T *__restrict__ x, T *__restrict__ out,
-                       int n_mats, int act, int out_act, long long M) {
+                       int n_mats, int out_act, long long M) {
     typedef Tile<T, W> TL;
     typedef typename Storage<T>::vec8 vec8;
-    constexpr int NK = TL::NK, NI = TL::NI;
+    constexpr int NK = TL::NK, NI = TL::NI, NF = TL::NF;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     vec8 *lds_w = reinterpret_cast<vec8 *>(smem_raw);
-    if (W_IN_LDS) stage_weights<T, W>(lds_w, wprep, n_mats);
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int j = lane & 31, h = lane >> 5;
@@ -72,25 +76,54 @@ __global__ void __launch_bounds__(kFwdThreads)
     const long long stride = (long long)gridDim.x * (blockDim.x >> 6);
     long long tile = (long long)blockIdx.x * (blockDim.x >> 6) + wave;
 
+    // the first tile is requested before the weights are staged, so both latencies overlap
     vec8 cur[NK];
     if (tile < n_tiles) TL::load(cur, x, tile * 32 + j, h, tile * 32 + j < M);
+    if (W_IN_LDS) stage_weights<T, W>(lds_w, wprep, n_mats);
+    const vec8 *wsrc = W_IN_LDS ? lds_w : wprep;
+
     while (tile < n_tiles) {
         const long long row = tile * 32 + j;
         const bool valid = row < M;
         // prefetch the next tile of this wave while the current one is being computed
         const long long next_tile = tile + stride;
         vec8 nxt[NK];
+#ifdef EXP_NO_LOAD
+        if (next_tile < n_tiles) { for (int kb = 0; kb < NK; ++kb) nxt[kb] = cur[kb]; }
+#else
         if (next_tile < n_tiles) TL::load(nxt, x, next_tile * 32 + j, h, next_tile * 32 + j < M);
+#endif
 
         if (STORE_INTERM) TL::store(cur, out, row, h, valid);
         f32x16 acc[NI];
-        for (int l = 0; l < n_mats - 1; ++l) {
-            TL::template matmul<W_IN_LDS>(acc, cur, lds_w, wprep, l, lane);
-            TL::repack_rt(cur, acc, act);
-            if (STORE_INTERM) TL::store(cur, out + (size_t)(l + 1) * M * W, row, h, valid);
+#ifdef EXP_NO_COMPUTE
+        if (n_mats < 0)
+#endif
+        if constexpr (NF <= 8 && PREFETCH) {
+            // all fragments of a matrix fit in registers: request matrix l+1 before converting layer l
+            vec8 frag[NF];
+            TL::load_frags(frag, wsrc, 0, lane);
+            for (int l = 0; l < n_mats - 1; ++l) {
+                TL::mma(acc, cur, frag);
+                TL::load_frags(frag, wsrc, l + 1, lane);
+                TL::template repack<ACT>(cur, acc);
+                if (STORE_INTERM) TL::store(cur, out + (size_t)(l + 1) * M * W, row, h, valid);
+            }
+            TL::mma(acc, cur, frag);
+        } else {
+            for (int l = 0; l < n_mats - 1; ++l) {
+                TL::template matmul<W_IN_LDS>(acc, cur, lds_w, wprep, l, lane);
+                TL::template repack<ACT>(cur, acc);
+                if (STORE_INTERM) TL::store(cur, out + (size_t)(l + 1) * M * W, row, h, valid);
+            }
+            TL::template matmul<W_IN_LDS>(acc, cur, lds_w, wprep, n_mats - 1, lane);
         }
-        TL::template matmul<W_IN_LDS>(acc, cur, lds_w, wprep, n_mats - 1, lane);
+#ifndef EXP_NO_COMPUTE
         TL::repack_rt(cur, acc, out_act);
+#endif
+#ifdef EXP_NO_STORE
+        if (cur[0][0] == (T)123.25f)
+#endif
         TL::store(cur, STORE_INTERM ? out + (size_t)n_mats * M * W : out, row, h, valid);
 
         if (next_tile < n_tiles) {
@@ -300,34 +333,85 @@ const DeviceInfo &device_info() {
 // LDS the weights may take and still leave room for two workgroups per CU.
 constexpr size_t kLdsBudget = 144 * 1024;
 
-template <typename T, int W, bool STORE_INTERM>
-static int launch_forward(const tnn_mlp_desc *d, const void *wprep, const void *x, void *out, size_t M, hipStream_t s) {
+// Grid of a streaming kernel: as many workgroups as the device holds at once (registers and LDS decide),
+// capped by the number of 32-row tiles. The result per kernel is cached.
+static long long stream_grid(const void *kernel, size_t lds_bytes, size_t M, int n_cu) {
+    struct Entry {
+        const void *k;
+        size_t lds;
+        int per_cu;
+    };
+    static thread_local Entry cache[64];
+    static thread_local int n_cache = 0;
+    int per_cu = 0;
+    for (int i = 0; i < n_cache; ++i)
+        if (cache[i].k == kernel && cache[i].lds == lds_bytes) per_cu = cache[i].per_cu;
+    if (!per_cu) {
+        int nb = 0;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, kernel, kFwdThreads, lds_bytes) != hipSuccess || nb < 1) {
+            (void)hipGetLastError();
+            nb = 1;
+        }
+        per_cu = nb;
+        if (n_cache < 64) cache[n_cache++] = Entry{kernel, lds_bytes, per_cu};
+    }
+    const long long n_tiles = ((long long)M + 31) / 32;
+    const int waves = kFwdThreads / 64;
+    long long blocks = (n_tiles + waves - 1) / waves;
+    if (blocks > (long long)n_cu * per_cu) blocks = (long long)n_cu * per_cu;
+    return blocks < 1 ? 1 : blocks;
+}
+
+template <typename T, int W, int ACT, bool STORE_INTERM, int THREADS, bool PREFETCH>
+static int launch_forward_v(const tnn_mlp_desc *d, const void *wprep, const void *x, void *out, size_t M, hipStream_t s, int per_cu) {
     typedef typename Storage<T>::vec8 vec8;
     const int n_mats = d->n_hidden_layers + 1;
     const size_t wbytes = prepared_elems(d) * sizeof(T);
     const DeviceInfo &di = device_info();
     if (!di.ok) return fail(TNN_ERR_HIP, "no usable HIP device");
-    const long long n_tiles = ((long long)M + 31) / 32;
-    const int waves = kFwdThreads / 64;
-    long long blocks = (n_tiles + waves - 1) / waves;
     const bool in_lds = wbytes <= kLdsBudget;
-    const int per_cu = (in_lds && wbytes > 72 * 1024) ? 1 : 2;
+    const long long n_tiles = ((long long)M + 31) / 32;
+    const int waves = THREADS / 64;
+    long long blocks = (n_tiles + waves - 1) / waves;
+    if (in_lds && wbytes * per_cu > 160 * 1024) per_cu = (int)(160 * 1024 / wbytes);
     if (blocks > (long long)di.n_cu * per_cu) blocks = (long long)di.n_cu * per_cu;
     if (blocks < 1) blocks = 1;
     if (in_lds) {
-        auto k = mlp_forward_kernel<T, W, STORE_INTERM, true>;
+        auto k = mlp_forward_kernel<T, W, ACT, STORE_INTERM, true, THREADS, PREFETCH>;
         if (wbytes > 48 * 1024 &&
             hipFuncSetAttribute(reinterpret_cast<const void *>(k), hipFuncAttributeMaxDynamicSharedMemorySize,
                                 (int)wbytes) != hipSuccess)
             return fail(TNN_ERR_HIP, "cannot reserve %zu bytes of LDS", wbytes);
-        hipLaunchKernelGGL(k, dim3((unsigned)blocks), dim3(kFwdThreads), wbytes, s, (const vec8 *)wprep, (const T *)x,
-                           (T *)out, n_mats, d->activation, d->output_activation, (long long)M);
+        hipLaunchKernelGGL(k, dim3((unsigned)blocks), dim3(THREADS), wbytes, s, (const vec8 *)wprep, (const T *)x,
+                           (T *)out, n_mats, d->output_activation, (long long)M);
     } else {
-        hipLaunchKernelGGL((mlp_forward_kernel<T, W, STORE_INTERM, false>), dim3((unsigned)blocks), dim3(kFwdThreads), 0,
-                           s, (const vec8 *)wprep, (const T *)x, (T *)out, n_mats, d->activation, d->output_activation,
-                           (long long)M);
+        auto k = mlp_forward_kernel<T, W, ACT, STORE_INTERM, false, THREADS, PREFETCH>;
+        hipLaunchKernelGGL(k, dim3((unsigned)blocks), dim3(THREADS), 0, s, (const vec8 *)wprep, (const T *)x, (T *)out,
+                           n_mats, d->output_activation, (long long)M);
     }
     return check_launch("mlp_forward_kernel");
+}
+
+template <typename T, int W, int ACT, bool STORE_INTERM>
+static int launch_forward_act(const tnn_mlp_desc *d, const void *wprep, const void *x, void *out, size_t M, hipStream_t s) {
+    static const char *ev = getenv("TNN_FWD_VARIANT");
+    const int v = ev ? atoi(ev) : 0;
+    switch (v) {
+    case 1: return launch_forward_v<T, W, ACT, STORE_INTERM, 512, true>(d, wprep, x, out, M, s, 2);
+    case 2: return launch_forward_v<T, W, ACT, STORE_INTERM, 256, true>(d, wprep, x, out, M, s, 3);
+    case 3: return launch_forward_v<T, W, ACT, STORE_INTERM, 256, false>(d, wprep, x, out, M, s, 4);
+    case 4: return launch_forward_v<T, W, ACT, STORE_INTERM, 256, false>(d, wprep, x, out, M, s, 3);
+    default: return launch_forward_v<T, W, ACT, STORE_INTERM, 512, false>(d, wprep, x, out, M, s, 2);
+    }
+}
+
+template <typename T, int W, bool STORE_INTERM>
+static int launch_forward(const tnn_mlp_desc *d, const void *wprep, const void *x, void *out, size_t M, hipStream_t s) {
+    switch (d->activation) {
+    case TNN_ACT_RELU: return launch_forward_act<T, W, TNN_ACT_RELU, STORE_INTERM>(d, wprep, x, out, M, s);
+    case TNN_ACT_SIGMOID: return launch_forward_act<T, W, TNN_ACT_SIGMOID, STORE_INTERM>(d, wprep, x, out, M, s);
+    default: return launch_forward_act<T, W, TNN_ACT_NONE, STORE_INTERM>(d, wprep, x, out, M, s);
+    }
 }
 
 template <typename T, int W>
@@ -338,23 +422,19 @@ static int launch_backward(const tnn_mlp_desc *d, const void *wprep_bwd, const v
     const size_t wbytes = prepared_elems(d) * sizeof(T);
     const DeviceInfo &di = device_info();
     if (!di.ok) return fail(TNN_ERR_HIP, "no usable HIP device");
-    const long long n_tiles = ((long long)M + 31) / 32;
-    const int waves = kFwdThreads / 64;
-    long long blocks = (n_tiles + waves - 1) / waves;
     const bool in_lds = wbytes <= kLdsBudget;
-    const int per_cu = (in_lds && wbytes > 72 * 1024) ? 1 : 2;
-    if (blocks > (long long)di.n_cu * per_cu) blocks = (long long)di.n_cu * per_cu;
-    if (blocks < 1) blocks = 1;
     if (in_lds) {
         auto k = mlp_backward_kernel<T, W, true>;
         if (wbytes > 48 * 1024 &&
             hipFuncSetAttribute(reinterpret_cast<const void *>(k), hipFuncAttributeMaxDynamicSharedMemorySize,
                                 (int)wbytes) != hipSuccess)
             return fail(TNN_ERR_HIP, "cannot reserve %zu bytes of LDS", wbytes);
+        const long long blocks = stream_grid(reinterpret_cast<const void *>(k), wbytes, M, di.n_cu);
         hipLaunchKernelGGL(k, dim3((unsigned)blocks), dim3(kFwdThreads), wbytes, s, (const vec8 *)wprep_bwd,
                            (const T *)dLdy, (const T *)interm_fwd, (T *)interm_bwd, (T *)dLdx, n_mats, d->activation,
                            d->output_activation, (long long)M);
     } else {
+        const long long blocks = stream_grid(reinterpret_cast<const void *>(mlp_backward_kernel<T, W, false>), 0, M, di.n_cu);
         hipLaunchKernelGGL((mlp_backward_kernel<T, W, false>), dim3((unsigned)blocks), dim3(kFwdThreads), 0, s,
                            (const vec8 *)wprep_bwd, (const T *)dLdy, (const T *)interm_fwd, (T *)interm_bwd, (T *)dLdx,
                            n_mats, d->activation, d->output_activation, (long long)M);

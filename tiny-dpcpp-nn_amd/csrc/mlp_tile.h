@@ -10,7 +10,8 @@
 
 namespace tnn {
 
-constexpr int kFwdThreads = 512; // 8 waves per workgroup share one LDS copy of the weights
+constexpr int kFwdThreads = 256;   // streaming kernels: 4 waves per workgroup share one LDS copy of the weights
+constexpr int kTrainThreads = 512; // fused training step: 8 waves per workgroup
 constexpr int kWaveSize = 64;
 
 // ------------------------------------------------------------------------------------------
@@ -23,30 +24,89 @@ template <int ACT> __device__ __forceinline__ float act_f32(float v) {
     return v;
 }
 
-// Accumulator half (8 fp32 of one 32x32 tile) -> activation -> 8 values of T.
-// ReLU before or after the rounding gives the same value (rounding keeps the sign).
-template <typename T, int ACT, int HALF>
-__device__ __forceinline__ typename Storage<T>::vec8 act_convert(const f32x16 &c) {
-    f32x8 v;
-#pragma unroll
-    for (int e = 0; e < 8; ++e) v[e] = act_f32<ACT>(c[HALF * 8 + e]);
-    return __builtin_convertvector(v, typename Storage<T>::vec8);
+typedef short s16x2 __attribute__((ext_vector_type(2)));
+typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+template <typename T> struct Pair;
+template <> struct Pair<bf16_t> { typedef bf16x2 type; };
+template <> struct Pair<fp16_t> { typedef fp16x2 type; };
+
+// Two fp32 -> one dword holding two values of T (round to nearest even): one packed convert.
+template <typename T> __device__ __forceinline__ unsigned int cvt_pair(float a, float b) {
+    const f32x2 v = {a, b};
+    return __builtin_bit_cast(unsigned int, __builtin_convertvector(v, typename Pair<T>::type));
 }
 
-// Backward: fp32 accumulator, masked / scaled by the stored forward activation, then rounded.
+// max(v, 0) on two 2-byte floats with one packed 16-bit integer instruction: a negative bf16/fp16 has
+// its sign bit set, i.e. is a negative int16, and every non-negative one is a non-negative int16.
+__device__ __forceinline__ unsigned int relu_pair(unsigned int v) {
+    const s16x2 b = __builtin_elementwise_max(__builtin_bit_cast(s16x2, v), s16x2{0, 0});
+    return __builtin_bit_cast(unsigned int, b);
+}
+
+// g where fwd > 0, else 0, with packed 16-bit integer instructions: m = min(max(fwd, 0), 1) is 1 exactly
+// for the positive values of fwd (as int16), and g * m keeps or clears the bit pattern of g. Written as
+// instructions because the compiler turns the 0/1 multiply back into per-half compares and selects.
+__device__ __forceinline__ unsigned int relu_gate_pair(unsigned int g, unsigned int fwd) {
+    unsigned int m, r;
+    const unsigned int zero = 0u, one = 0x00010001u;
+    asm("v_pk_max_i16 %0, %1, %2" : "=v"(m) : "v"(fwd), "v"(zero));
+    asm("v_pk_min_i16 %0, %1, %2" : "=v"(m) : "v"(m), "v"(one));
+    asm("v_pk_mul_lo_u16 %0, %1, %2" : "=v"(r) : "v"(g), "v"(m));
+    return r;
+}
+
+// The same gate when fwd is known to be the output of relu_pair (never negative, never -0): min(fwd, 1)
+// as unsigned 16-bit integers is already the 0/1 mask.
+__device__ __forceinline__ unsigned int relu_gate_pair_nonneg(unsigned int g, unsigned int fwd) {
+    unsigned int m, r;
+    const unsigned int one = 0x00010001u;
+    asm("v_pk_min_u16 %0, %1, %2" : "=v"(m) : "v"(fwd), "v"(one));
+    asm("v_pk_mul_lo_u16 %0, %1, %2" : "=v"(r) : "v"(g), "v"(m));
+    return r;
+}
+
+// Accumulator half (8 fp32 of one 32x32 tile) -> activation -> 8 values of T.
+// ReLU before or after the rounding gives the same value (rounding keeps the sign), so it is applied to
+// the rounded values, two per instruction.
 template <typename T, int ACT, int HALF>
+__device__ __forceinline__ typename Storage<T>::vec8 act_convert(const f32x16 &c) {
+    u32x4 r;
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+        float a = c[HALF * 8 + 2 * p], b = c[HALF * 8 + 2 * p + 1];
+        if (ACT == TNN_ACT_SIGMOID) {
+            a = act_f32<ACT>(a);
+            b = act_f32<ACT>(b);
+        }
+        unsigned int u = cvt_pair<T>(a, b);
+        if (ACT == TNN_ACT_RELU) u = relu_pair(u);
+        r[p] = u;
+    }
+    return __builtin_bit_cast(typename Storage<T>::vec8, r);
+}
+
+// Backward: fp32 accumulator, masked / scaled by the stored forward activation, then rounded
+// (zeroing before or after the rounding is the same). NONNEG: the activation was produced by this
+// library's own ReLU in the same kernel.
+template <typename T, int ACT, int HALF, bool NONNEG = false>
 __device__ __forceinline__ typename Storage<T>::vec8 bwd_convert(const f32x16 &c,
                                                                  const typename Storage<T>::vec8 &fwd) {
-    f32x8 v;
+    const u32x4 fw = __builtin_bit_cast(u32x4, fwd);
+    u32x4 r;
 #pragma unroll
-    for (int e = 0; e < 8; ++e) {
-        float t = c[HALF * 8 + e];
-        const float f = (float)fwd[e];
-        if (ACT == TNN_ACT_RELU) t = (f <= 0.0f) ? 0.0f : t;
-        if (ACT == TNN_ACT_SIGMOID) t = as_fp32(t * (f * (1.0f - f)));
-        v[e] = t;
+    for (int p = 0; p < 4; ++p) {
+        float a = c[HALF * 8 + 2 * p], b = c[HALF * 8 + 2 * p + 1];
+        if (ACT == TNN_ACT_SIGMOID) {
+            const float fa = (float)fwd[2 * p], fb = (float)fwd[2 * p + 1];
+            a = as_fp32(a * (fa * (1.0f - fa)));
+            b = as_fp32(b * (fb * (1.0f - fb)));
+        }
+        unsigned int u = cvt_pair<T>(a, b);
+        if (ACT == TNN_ACT_RELU) u = NONNEG ? relu_gate_pair_nonneg(u, fw[p]) : relu_gate_pair(u, fw[p]);
+        r[p] = u;
     }
-    return __builtin_convertvector(v, typename Storage<T>::vec8);
+    return __builtin_bit_cast(typename Storage<T>::vec8, r);
 }
 
 template <typename T, int W> struct Tile {
@@ -72,6 +132,26 @@ template <typename T, int W> struct Tile {
         if (valid) {
 #pragma unroll
             for (int kb = 0; kb < NK; ++kb) p[2 * kb] = r[kb];
+        }
+    }
+
+    static constexpr int NF = NI * NK; // weight fragments per matrix and lane
+
+    // The lane's NF operand fragments of matrix l (LDS or global, already in operand order).
+    static __device__ __forceinline__ void load_frags(vec8 (&f)[NF], const vec8 *__restrict__ w, int l, int lane) {
+        const vec8 *p = w + (size_t)l * (NF * kWaveSize) + lane;
+#pragma unroll
+        for (int i = 0; i < NF; ++i) f[i] = p[i * kWaveSize];
+    }
+
+    // acc[a] = sum_kb frag(a, kb) * b[kb]
+    static __device__ __forceinline__ void mma(f32x16 (&acc)[NI], const vec8 (&b)[NK], const vec8 (&f)[NF]) {
+#pragma unroll
+        for (int a = 0; a < NI; ++a) acc[a] = f32x16{};
+#pragma unroll
+        for (int kb = 0; kb < NK; ++kb) {
+#pragma unroll
+            for (int a = 0; a < NI; ++a) acc[a] = Storage<T>::mfma(f[a * NK + kb], b[kb], acc[a]);
         }
     }
 
@@ -108,12 +188,12 @@ template <typename T, int W> struct Tile {
             repack<TNN_ACT_NONE>(r, acc);
     }
 
-    template <int ACT>
+    template <int ACT, bool NONNEG = false>
     static __device__ __forceinline__ void bwd_repack(vec8 (&r)[NK], const f32x16 (&acc)[NI], const vec8 (&fwd)[NK]) {
 #pragma unroll
         for (int a = 0; a < NI; ++a) {
-            r[2 * a] = bwd_convert<T, ACT, 0>(acc[a], fwd[2 * a]);
-            if (2 * a + 1 < NK) r[2 * a + 1] = bwd_convert<T, ACT, 1>(acc[a], fwd[2 * a + 1 < NK ? 2 * a + 1 : 0]);
+            r[2 * a] = bwd_convert<T, ACT, 0, NONNEG>(acc[a], fwd[2 * a]);
+            if (2 * a + 1 < NK) r[2 * a + 1] = bwd_convert<T, ACT, 1, NONNEG>(acc[a], fwd[2 * a + 1 < NK ? 2 * a + 1 : 0]);
         }
     }
 };

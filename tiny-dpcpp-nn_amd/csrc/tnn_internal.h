@@ -40,7 +40,7 @@ typedef _Float16 fp16x4 __attribute__((ext_vector_type(4)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef _Float16 fp16x2 __attribute__((ext_vector_type(2)));
 
-// Per storage type: 8-wide vector, and the 32x32x16 MFMA (fp32 accumulate).
+// Per storage type: 8-wide vector, the 32x32x16 MFMA and the 16x16x32 MFMA (fp32 accumulate).
 template <typename T> struct Storage;
 template <> struct Storage<bf16_t> {
     typedef bf16x8 vec8;
@@ -48,12 +48,18 @@ template <> struct Storage<bf16_t> {
     static __device__ __forceinline__ f32x16 mfma(vec8 a, vec8 b, f32x16 c) {
         return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
     }
+    static __device__ __forceinline__ f32x4 mfma16(vec8 a, vec8 b, f32x4 c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+    }
 };
 template <> struct Storage<fp16_t> {
     typedef fp16x8 vec8;
     typedef fp16x4 vec4;
     static __device__ __forceinline__ f32x16 mfma(vec8 a, vec8 b, f32x16 c) {
         return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ f32x4 mfma16(vec8 a, vec8 b, f32x4 c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
     }
 };
 

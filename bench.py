@@ -167,9 +167,7 @@ def main():
                                            ptr(ws), ws_bytes, s)
             if timed >= 0:
                 ke[timed].record()
-            rc |= lib.tnn_pack_and_transpose(FP32, W, n_mats, ptr(dW), ptr(dWp), s)
-            rc |= lib.tnn_adam_step(ptr(master), ptr(m), ptr(v), ptr(dWp), FP32, 1.0, master.numel(), i + 1, 1e-3, 0.9, 0.99, 1e-15, None, BF16, s)
-            rc |= lib.tnn_mlp_prepare_weights(d, ptr(master), 1, ptr(pf), ptr(pb), s)
+            rc |= lib.tnn_mlp_adam_update(d, ptr(master), ptr(m), ptr(v), ptr(dW), 1.0, i + 1, 1e-3, 0.9, 0.99, 1e-15, None, ptr(pf), ptr(pb), s)
             if rc:
                 raise RuntimeError(lib.tnn_last_error())
 

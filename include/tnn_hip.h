@@ -169,6 +169,19 @@ int tnn_adam_step(float *d_param, float *d_m, float *d_v, const void *d_grad, in
                   size_t n, int step, float lr, float beta1, float beta2, float eps, void *d_param_T,
                   int param_T_dtype, tnn_stream_t stream);
 
+/* The optimizer step of a training loop on the fused MLP in one launch: what the reference's loop does
+ * with PackAndTranspose of the raw gradients (include/tnn_api.h:599-603), torch.optim.Adam on the packed fp32
+ * parameter (dpcpp_bindings/tiny_dpcpp_nn/modules.py:171-175) and set_params (modules.py:184-207, which
+ * re-derives the device copies on every forward). Identical, bit for bit, to tnn_pack_and_transpose +
+ * tnn_adam_step + tnn_mlp_prepare_weights.
+ *   d_master_packed, d_m, d_v: fp32, packed parameter layout. d_dW_raw: fp32 [out][in] as written by
+ *   tnn_mlp_backward / tnn_mlp_train_step_l2 with dW_is_fp32 != 0; multiplied by grad_scale (1/loss_scale).
+ *   d_packed_T (may be NULL): updated parameters rounded to T, packed layout. d_prepared_fwd / d_prepared_bwd
+ *   (may be NULL): the operand-order copies, updated in place. */
+int tnn_mlp_adam_update(const tnn_mlp_desc *desc, float *d_master_packed, float *d_m, float *d_v, const float *d_dW_raw,
+                        float grad_scale, int step, float lr, float beta1, float beta2, float eps, void *d_packed_T,
+                        void *d_prepared_fwd, void *d_prepared_bwd, tnn_stream_t stream);
+
 /* ------------------------------------------------------------------------------------------
  * Multi-resolution hash grid (include/encodings/grid.h, include/common/common_device.h:700-775).
  * ------------------------------------------------------------------------------------------ */

@@ -42,7 +42,11 @@ def test_descriptor_validation_is_host_only(lib):
         assert lib.tnn_mlp_prepared_bytes(ctypes.byref(bad)) == 0
         assert lib.tnn_mlp_backward_workspace_bytes(ctypes.byref(bad), 1024) == 0
     assert lib.tnn_mlp_backward_workspace_bytes(ctypes.byref(good), 1 << 18) > 0
-    assert lib.tnn_mlp_train_step_workspace_bytes(ctypes.byref(good), 1 << 18) > lib.tnn_mlp_backward_workspace_bytes(ctypes.byref(good), 1 << 18)
+    # the fused training step only needs room for per-workgroup partial weight gradients ...
+    assert 0 < lib.tnn_mlp_train_step_workspace_bytes(ctypes.byref(good), 1 << 18) < 64 << 20
+    # ... wider networks stage activations and deltas in the workspace
+    wide = _lib.MlpDesc(_lib.TNN_FP16, 128, 8, _lib.ACT_RELU, _lib.ACT_NONE)
+    assert lib.tnn_mlp_train_step_workspace_bytes(ctypes.byref(wide), 1 << 18) > lib.tnn_mlp_backward_workspace_bytes(ctypes.byref(wide), 1 << 18)
 
 
 def test_grid_descriptor_host_side(lib):

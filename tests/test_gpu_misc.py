@@ -53,3 +53,35 @@ def test_adam(tnn, oracle):
     tnn.adam_step(p, m, v, torch.from_numpy(g16).to(tnn.dev).to(torch.bfloat16), BF16, 1.0, 5, 1e-3, 0.9, 0.99, 1e-15)
     rp, rm, rv = oracle.adam_step(rp, rm, rv, g16, 5, 1e-3, 0.9, 0.99, 1e-15)
     assert np.allclose(tnn.host(p), rp, rtol=1e-6, atol=1e-7)
+
+
+@pytest.mark.parametrize("dtype,tdt", [(BF16, torch.bfloat16), (FP16, torch.float16)])
+@pytest.mark.parametrize("W,n_hidden", [(64, 4), (16, 2), (32, 3), (128, 1)])
+def test_fused_adam_update_equals_the_three_separate_calls(tnn, dtype, tdt, W, n_hidden):
+    """tnn_mlp_adam_update == tnn_pack_and_transpose + tnn_adam_step + tnn_mlp_prepare_weights, bit for bit."""
+    import ctypes
+    from gpu_harness import ptr
+    from tiny_dpcpp_nn import _lib
+    n_mats = n_hidden + 1
+    n = n_mats * W * W
+    gen = torch.Generator(device=tnn.dev).manual_seed(W + n_hidden)
+    desc = tnn.mlp_desc(dtype, W, n_hidden, "relu", "none")
+    master = torch.randn(n, device=tnn.dev, generator=gen) * 0.1
+    m0 = torch.randn(n, device=tnn.dev, generator=gen) * 0.01
+    v0 = torch.rand(n, device=tnn.dev, generator=gen) * 0.01
+    dW = torch.randn((n_mats, W, W), device=tnn.dev, generator=gen)
+    # separate calls
+    p1, m1, v1 = master.clone(), m0.clone(), v0.clone()
+    gp = torch.empty(n, device=tnn.dev)
+    _lib.check(tnn.lib.tnn_pack_and_transpose(FP32, W, n_mats, ptr(dW), ptr(gp), tnn.stream()))
+    pT1 = torch.empty(n, dtype=tdt, device=tnn.dev)
+    tnn.adam_step(p1, m1, v1, gp, FP32, 1.0 / 128, 3, 1e-3, 0.9, 0.99, 1e-15, pT1, dtype)
+    f1, b1 = tnn.prepare_packed(desc, p1, src_is_fp32=True)
+    # one call; the operand buffers start from a prepared state (their zero padding is never rewritten)
+    p2, m2, v2 = master.clone(), m0.clone(), v0.clone()
+    f2, b2 = tnn.prepare_packed(desc, master, src_is_fp32=True)
+    pT2 = torch.empty(n, dtype=tdt, device=tnn.dev)
+    _lib.check(tnn.lib.tnn_mlp_adam_update(ctypes.byref(desc), ptr(p2), ptr(m2), ptr(v2), ptr(dW), 1.0 / 128, 3, 1e-3, 0.9, 0.99, 1e-15,
+                                           ptr(pT2), ptr(f2), ptr(b2), tnn.stream()))
+    for a, b in ((p1, p2), (m1, m2), (v1, v2), (pT1, pT2), (f1, f2), (b1, b2)):
+        assert torch.equal(a, b)

@@ -87,6 +87,11 @@ SIGNATURES = {
         [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_float, c_size_t, c_int, c_float, c_float, c_float, c_float, c_void_p,
          c_int, c_void_p],
     ),
+    "tnn_mlp_adam_update": (
+        c_int,
+        [POINTER(MlpDesc), c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_int, c_float, c_float, c_float, c_float, c_void_p,
+         c_void_p, c_void_p, c_void_p],
+    ),
     "tnn_grid_desc_init": (
         c_int,
         [POINTER(GridDesc), c_uint32, c_uint32, c_uint32, c_uint32, c_uint32, c_float, c_uint32, c_uint32, c_uint32, c_uint32],

@@ -73,6 +73,12 @@ int tnn_abi_version(void);
 /* Number of HIP devices whose architecture is gfx950, or a negative status. */
 int tnn_device_check(void);
 
+/* DeviceMatrix::fill / DeviceMatrices::fill (include/common/DeviceMatrix.h:167,381): n elements of dtype := value. */
+int tnn_fill(int dtype, void *d_ptr, size_t n, float value, tnn_stream_t stream);
+/* DeviceMatrix::copy_from_device / DeviceMem::copy_from_device (include/common/DeviceMatrix.h:198-201,
+ * include/common/DeviceMem.h:91-95): element-wise type-converting copy (round to nearest even). */
+int tnn_cast(int dst_dtype, void *d_dst, int src_dtype, const void *d_src, size_t n, tnn_stream_t stream);
+
 /* ------------------------------------------------------------------------------------------
  * Weight layouts.
  *   unpacked : per matrix element (k=in, n=out) at k*W + n (test/mlp.h:391-402)

@@ -133,60 +133,109 @@ template <typename O> __device__ __forceinline__ O to_out(float v) { return (O)v
 
 constexpr int kGridThreads = 256;
 
+// Levels are processed in groups whose outputs fill one 16-byte piece of the encoded row: all gathers of a
+// group (GL * 2^D independent loads) are issued before the first blend, and the row is written in whole
+// 16-byte pieces (a per-level 4-byte store turns into a 32-byte masked write at the memory controller).
 template <int D, int F, typename P, typename O>
 __global__ void __launch_bounds__(kGridThreads)
     grid_forward_kernel(const GridLevels lv, const GridParams gp, const float *__restrict__ xin, const P *__restrict__ table,
                         O *__restrict__ out, long long M) {
+    constexpr int PER16 = 16 / (int)sizeof(O);            // outputs per 16-byte piece
+    constexpr int GL = (PER16 / F) > 0 ? (PER16 / F) : 1; // levels per group (F = 8 with fp32 output: 1 level, 2 pieces)
+    constexpr int NOUT = GL * F;
+    typedef O ovec __attribute__((ext_vector_type(NOUT)));
     const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= M) return;
     float x[D];
 #pragma unroll
     for (int d = 0; d < D; ++d) x[d] = xin[i * D + d];
     O *orow = out + i * gp.padded_width;
+    const bool row_aligned = ((gp.padded_width * sizeof(O)) % 16 == 0) && ((reinterpret_cast<uintptr_t>(out) & 15) == 0);
 
-    for (uint32_t l = 0; l < gp.n_levels; ++l) {
-        const uint32_t size = lv.size[l], res = lv.resolution[l], flags = lv.flags[l];
-        const P *g = table + (size_t)lv.offset[l] * F;
-        uint32_t cell[D];
-        float frac[D];
-        cell_of<D>(x, lv.scale[l], gp.interpolation, cell, frac);
-        float result[F];
-        if (gp.interpolation == TNN_INTERP_NEAREST) {
-            const uint32_t idx = level_index<D>(cell, size, res, flags, gp.hash_type);
-            load_entry<P, F>(g + (size_t)idx * F, result);
-        } else {
-            float vals[1 << D][F];
-            float wts[1 << D];
+    for (uint32_t l0 = 0; l0 < gp.n_levels; l0 += GL) {
+        float vals[GL][1 << D][F];
+        float wts[GL][1 << D];
+        // gathers of the whole group
 #pragma unroll
-            for (int c = 0; c < (1 << D); ++c) {
-                float weight = 1.0f;
-                uint32_t loc[D];
+        for (int gl = 0; gl < GL; ++gl) {
+            const uint32_t l = l0 + gl;
+            if (l < gp.n_levels) {
+                const uint32_t size = lv.size[l], res = lv.resolution[l], flags = lv.flags[l];
+                const P *g = table + (size_t)lv.offset[l] * F;
+                uint32_t cell[D];
+                float frac[D];
+                cell_of<D>(x, lv.scale[l], gp.interpolation, cell, frac);
+                if (gp.interpolation == TNN_INTERP_NEAREST) {
+                    const uint32_t idx = level_index<D>(cell, size, res, flags, gp.hash_type);
+                    load_entry<P, F>(g + (size_t)idx * F, vals[gl][0]);
+                    wts[gl][0] = 1.0f;
 #pragma unroll
-                for (int d = 0; d < D; ++d) {
-                    if ((c & (1 << d)) == 0) {
-                        weight *= 1 - frac[d];
-                        loc[d] = cell[d];
-                    } else {
-                        weight *= frac[d];
-                        loc[d] = cell[d] + 1;
+                    for (int c = 1; c < (1 << D); ++c) {
+                        wts[gl][c] = 0.0f;
+#pragma unroll
+                        for (int f = 0; f < F; ++f) vals[gl][c][f] = 0.0f;
+                    }
+                } else {
+#pragma unroll
+                    for (int c = 0; c < (1 << D); ++c) {
+                        float weight = 1.0f;
+                        uint32_t loc[D];
+#pragma unroll
+                        for (int d = 0; d < D; ++d) {
+                            if ((c & (1 << d)) == 0) {
+                                weight *= 1 - frac[d];
+                                loc[d] = cell[d];
+                            } else {
+                                weight *= frac[d];
+                                loc[d] = cell[d] + 1;
+                            }
+                        }
+                        wts[gl][c] = weight;
+                        const uint32_t idx = level_index<D>(loc, size, res, flags, gp.hash_type);
+                        load_entry<P, F>(g + (size_t)idx * F, vals[gl][c]);
                     }
                 }
-                wts[c] = weight;
-                const uint32_t idx = level_index<D>(loc, size, res, flags, gp.hash_type);
-                load_entry<P, F>(g + (size_t)idx * F, vals[c]);
             }
-#pragma unroll
-            for (int f = 0; f < F; ++f) result[f] = 0.0f;
-            // same corner order and fused multiply-add as include/encodings/grid.h:114-129
-#pragma unroll
-            for (int c = 0; c < (1 << D); ++c)
-#pragma unroll
-                for (int f = 0; f < F; ++f) result[f] = __builtin_fmaf(wts[c], vals[c][f], result[f]);
         }
+        // blends, in the corner order and with the fused multiply-add of include/encodings/grid.h:114-129
+        // (nearest: the single value is copied, grid.h:104-109)
+        ovec o;
 #pragma unroll
-        for (int f = 0; f < F; ++f) orow[l * F + f] = to_out<O>(result[f]);
+        for (int gl = 0; gl < GL; ++gl) {
+#pragma unroll
+            for (int f = 0; f < F; ++f) {
+                float r = 0.0f;
+                if (gp.interpolation == TNN_INTERP_NEAREST) {
+                    r = vals[gl][0][f];
+                } else {
+#pragma unroll
+                    for (int c = 0; c < (1 << D); ++c) r = __builtin_fmaf(wts[gl][c], vals[gl][c][f], r);
+                }
+                o[gl * F + f] = to_out<O>(r);
+            }
+        }
+        const uint32_t col0 = l0 * F;
+        if (row_aligned && l0 + GL <= gp.n_levels) {
+            if constexpr (NOUT * sizeof(O) == 16) {
+                *reinterpret_cast<ovec *>(orow + col0) = o;
+            } else { // F = 8 with fp32 output: two 16-byte pieces
+#pragma unroll
+                for (int e = 0; e < NOUT; ++e) orow[col0 + e] = o[e];
+            }
+        } else {
+#pragma unroll
+            for (int e = 0; e < NOUT; ++e)
+                if (l0 + e / F < gp.n_levels) orow[col0 + e] = o[e];
+        }
     }
-    for (uint32_t c = gp.n_levels * F; c < gp.padded_width; ++c) orow[c] = to_out<O>(0.0f);
+    // zero padding of the row (include/encodings/grid.h:682-694), in 16-byte pieces where the row allows it
+    uint32_t c = gp.n_levels * F;
+    if (row_aligned) {
+        typedef O zvec __attribute__((ext_vector_type(PER16)));
+        for (; c < gp.padded_width && (c % PER16) != 0; ++c) orow[c] = to_out<O>(0.0f);
+        for (; c + PER16 <= gp.padded_width; c += PER16) *reinterpret_cast<zvec *>(orow + c) = zvec{};
+    }
+    for (; c < gp.padded_width; ++c) orow[c] = to_out<O>(0.0f);
 }
 
 template <int D>

@@ -110,6 +110,14 @@ __global__ void adam_kernel(float *__restrict__ param, float *__restrict__ m, fl
     if (param_T) param_T[i] = (P)p;
 }
 
+template <typename T> __global__ void fill_kernel(T *__restrict__ p, size_t n, T v) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) p[i] = v;
+}
+
+template <typename D, typename S> __global__ void cast_kernel(D *__restrict__ d, const S *__restrict__ s, size_t n) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) d[i] = (D)(float)s[i];
+}
+
 // One thread per weight: reads the raw gradient element dW[l][n][k], updates the fp32 master copy (packed
 // layout) with Adam, and writes the rounded weight to the packed T copy and to both operand-order copies.
 template <typename T>
@@ -283,4 +291,43 @@ TNN_API int tnn_mlp_adam_update(const tnn_mlp_desc *desc, float *d_master_packed
                            grad_scale, W, n_mats, step_size, bc2_sqrt, beta1, beta2, eps, (fp16_t *)d_packed_T, (fp16_t *)d_prepared_fwd,
                            (fp16_t *)d_prepared_bwd);
     return check_launch("mlp_adam_update_kernel");
+}
+
+TNN_API int tnn_fill(int dtype, void *d_ptr, size_t n, float value, tnn_stream_t stream) {
+    if (!d_ptr && n) return fail(TNN_ERR_INVALID_ARGUMENT, "NULL pointer argument");
+    if (n == 0) return TNN_OK;
+    size_t blocks = (n + 255) / 256;
+    if (blocks > 8192) blocks = 8192;
+    hipStream_t s = as_stream(stream);
+    switch (dtype) {
+    case TNN_BF16: hipLaunchKernelGGL((fill_kernel<bf16_t>), dim3((unsigned)blocks), dim3(256), 0, s, (bf16_t *)d_ptr, n, (bf16_t)value); break;
+    case TNN_FP16: hipLaunchKernelGGL((fill_kernel<fp16_t>), dim3((unsigned)blocks), dim3(256), 0, s, (fp16_t *)d_ptr, n, (fp16_t)value); break;
+    case TNN_FP32: hipLaunchKernelGGL((fill_kernel<float>), dim3((unsigned)blocks), dim3(256), 0, s, (float *)d_ptr, n, value); break;
+    default: return fail(TNN_ERR_UNSUPPORTED, "dtype %d", dtype);
+    }
+    return check_launch("fill_kernel");
+}
+
+template <typename D> static int launch_cast(D *d, int src_dtype, const void *src, size_t n, hipStream_t s) {
+    size_t blocks = (n + 255) / 256;
+    if (blocks > 8192) blocks = 8192;
+    switch (src_dtype) {
+    case TNN_BF16: hipLaunchKernelGGL((cast_kernel<D, bf16_t>), dim3((unsigned)blocks), dim3(256), 0, s, d, (const bf16_t *)src, n); break;
+    case TNN_FP16: hipLaunchKernelGGL((cast_kernel<D, fp16_t>), dim3((unsigned)blocks), dim3(256), 0, s, d, (const fp16_t *)src, n); break;
+    case TNN_FP32: hipLaunchKernelGGL((cast_kernel<D, float>), dim3((unsigned)blocks), dim3(256), 0, s, d, (const float *)src, n); break;
+    default: return fail(TNN_ERR_UNSUPPORTED, "src dtype %d", src_dtype);
+    }
+    return check_launch("cast_kernel");
+}
+
+TNN_API int tnn_cast(int dst_dtype, void *d_dst, int src_dtype, const void *d_src, size_t n, tnn_stream_t stream) {
+    if ((!d_dst || !d_src) && n) return fail(TNN_ERR_INVALID_ARGUMENT, "NULL pointer argument");
+    if (n == 0) return TNN_OK;
+    hipStream_t s = as_stream(stream);
+    switch (dst_dtype) {
+    case TNN_BF16: return launch_cast<bf16_t>((bf16_t *)d_dst, src_dtype, d_src, n, s);
+    case TNN_FP16: return launch_cast<fp16_t>((fp16_t *)d_dst, src_dtype, d_src, n, s);
+    case TNN_FP32: return launch_cast<float>((float *)d_dst, src_dtype, d_src, n, s);
+    default: return fail(TNN_ERR_UNSUPPORTED, "dst dtype %d", dst_dtype);
+    }
 }

@@ -61,6 +61,8 @@ SIGNATURES = {
     "tnn_last_error": (c_char_p, []),
     "tnn_abi_version": (c_int, []),
     "tnn_device_check": (c_int, []),
+    "tnn_fill": (c_int, [c_int, c_void_p, c_size_t, c_float, c_void_p]),
+    "tnn_cast": (c_int, [c_int, c_void_p, c_int, c_void_p, c_size_t, c_void_p]),
     "tnn_pack_weights": (c_int, [c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]),
     "tnn_unpack_weights": (c_int, [c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]),
     "tnn_packed_transpose": (c_int, [c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]),

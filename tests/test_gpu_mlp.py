@@ -158,7 +158,7 @@ def test_closed_forms(tnn, oracle):
     desc = tnn.mlp_desc(dtype, W, n_hidden, "none", "none")
     _, pf, pb = tnn.prepare(desc, w)
     interm = tnn.host(tnn.forward(desc, pf, tnn.dev_tensor(x, dtype)))
-    c = float(oracle.round(np.float32(0.01), dtype))
+    c = float(oracle.round(np.float32([0.01]), dtype)[0])
     assert np.allclose(interm[1], c * n_in, rtol=1e-2)
     assert np.allclose(interm[2], c * n_in * W * c, rtol=1e-2)
     assert np.allclose(interm[3][:, :n_out], c * n_in * W * c * W * c, rtol=2e-2)
@@ -168,7 +168,7 @@ def test_closed_forms(tnn, oracle):
         n_hidden, B = 4, 64
         n_mats = n_hidden + 1
         w = np.full((n_mats, W, W), 1.0 / W)
-        v = float(oracle.round(np.float32(np.sqrt(1.0 / B)), dtype))
+        v = float(oracle.round(np.float32([np.sqrt(1.0 / B)]), dtype)[0])
         desc = tnn.mlp_desc(dtype, W, n_hidden, "none", "none")
         _, pf, pb = tnn.prepare(desc, w)
         xt = tnn.dev_tensor(np.full((B, W), v), dtype)

@@ -1,0 +1,317 @@
+"""GPU tests of the Python package (tiny_dpcpp_nn.Network / Encoding / NetworkWithInputEncoding).
+
+They follow the reference's Python tests: forward and gradients against an fp32 linear stack built from the same
+weights (test/python/test_compare_torch_dpcpp.py:92-157,185-242), set/get params (test_set_param.py:48-61),
+zeroed padding weights (test_padding_bias.py:176-213), output shapes of encodings (test_encodings.py:607-608), and
+a short training run (test_training.py). Network results are also checked against the CPU oracle, which rounds
+where the kernels round.
+
+Tolerances: tests/tolerances.py (bf16 1e-2 rel / 1e-3 abs, fp16 5e-3 rel / 5e-4 abs; end to end "propagated").
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle_bindings import BF16, FP16
+from tolerances import assert_propagated, max_norm_rel
+
+pytestmark = pytest.mark.gpu
+
+DEVICE = "cuda"
+DT = {torch.float16: FP16, torch.bfloat16: BF16}
+
+
+@pytest.fixture(scope="module")
+def tcnn():
+    import tiny_dpcpp_nn
+
+    assert torch.cuda.is_available(), "these tests need the GPU"
+    return tiny_dpcpp_nn
+
+
+def net_config(width, n_hidden, act="relu", out_act="none"):
+    return {"otype": "FullyFusedMLP", "activation": act, "output_activation": out_act, "n_neurons": width, "n_hidden_layers": n_hidden}
+
+
+def packed_index(width):
+    """perm[k * W + n] = position of element (k=in, n=out) inside one packed matrix."""
+    k, n = np.divmod(np.arange(width * width), width)
+    return (k & ~1) * width + 2 * n + (k & 1)
+
+
+def unpack(packed, n_mats, width):
+    """Packed parameter vector -> (n_mats, W, W) array indexed [matrix][in][out]."""
+    p = np.asarray(packed, np.float32).reshape(n_mats, width * width)
+    return p[:, packed_index(width)].reshape(n_mats, width, width)
+
+
+def random_weights(n_mats, width, seed, dtype):
+    g = torch.Generator().manual_seed(seed)
+    bound = (6.0 / (2 * width)) ** 0.5
+    w = (torch.rand(n_mats, width, width, generator=g) * 2 - 1) * bound
+    return w.to(dtype).to(torch.float32)  # values representable in dtype
+
+
+def torch_reference(x_padded, weights, act, out_act):
+    """fp32 autograd reference: y = f_out(f(...f(x W_0)...) W_L) with [in][out] matrices."""
+    fns = {"relu": torch.relu, "sigmoid": torch.sigmoid, "none": lambda t: t}
+    h = x_padded
+    for i, w in enumerate(weights):
+        h = h @ w
+        h = fns[out_act if i == len(weights) - 1 else act](h)
+    return h
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("width,n_hidden,n_in,n_out,act,out_act,use_bias,batch", [
+    (64, 4, 64, 64, "relu", "none", False, 1024),
+    (64, 2, 32, 3, "relu", "none", True, 512),
+    (16, 2, 16, 16, "sigmoid", "none", False, 64),
+    (32, 3, 5, 7, "none", "sigmoid", True, 13),       # ragged batch: padded to 16 rows inside
+    (128, 2, 100, 128, "relu", "relu", False, 40),
+])
+def test_network_forward_and_gradients(tcnn, oracle, dtype, width, n_hidden, n_in, n_out, act, out_act, use_bias, batch):
+    torch.manual_seed(0)
+    n_mats = n_hidden + 1
+    net = tcnn.Network(n_in, n_out, net_config(width, n_hidden, act, out_act), dtype=dtype, use_bias=use_bias)
+    assert net.params.dtype == torch.float32 and net.params.numel() == n_mats * width * width
+    assert net.loss_scale == (128.0 if dtype == torch.float16 else 1.0)
+
+    w = random_weights(n_mats, width, 42, dtype)
+    net.set_params(w.reshape(-1).to(DEVICE))
+
+    # what the module holds: packed; rows of W_0 beyond the one-padded input width and columns of W_L beyond n_out are zero
+    # (include/network/Network.h:182-203 of the reference: with use_bias an input width that already is a multiple of 16
+    # keeps every row, the ones the module pads with then reach all of them)
+    one_padded = n_in if not use_bias else (width if n_in % 16 == 0 else ((n_in + 15) // 16) * 16)
+    w_eff = w.clone()
+    w_eff[0, one_padded:, :] = 0
+    w_eff[-1, :, n_out:] = 0
+    held = unpack(net.get_params().float().cpu().numpy().reshape(-1), n_mats, width)
+    np.testing.assert_array_equal(held, w_eff.numpy())
+    np.testing.assert_array_equal(unpack(net.params.detach().cpu().numpy().reshape(-1), n_mats, width), w_eff.numpy())
+
+    x = (torch.rand(batch, n_in) * 2 - 1).to(dtype)
+    x_dev = x.to(DEVICE).requires_grad_(True)
+    x_pad = torch.nn.functional.pad(x.float(), [0, width - n_in], value=float(use_bias))
+
+    # ---- eval mode: the inference kernel
+    net.eval()
+    with torch.no_grad():
+        y_eval = net(x_dev)
+    assert y_eval.shape == (batch, n_out) and y_eval.dtype == dtype
+    n_rows = ((batch + 7) // 8) * 8
+    x_or = np.zeros((n_rows, width), np.float32)
+    x_or[:batch] = x_pad.numpy()
+    interm = oracle.mlp_forward_T(DT[dtype], width, n_mats, act, out_act, w_eff.numpy(), x_or)
+    y_oracle = interm[-1][:batch, :n_out]
+    assert_propagated(y_eval.float().cpu().numpy(), y_oracle, DT[dtype], "inference vs oracle")
+
+    # ---- train mode: forward that keeps activations, then backward through autograd
+    net.train()
+    y = net(x_dev)
+    assert y.shape == (batch, n_out)
+    np.testing.assert_array_equal(y.detach().float().cpu().numpy(), y_eval.float().cpu().numpy())
+    g = ((torch.rand(batch, n_out) * 2 - 1) / batch).to(dtype)
+    y.backward(g.to(DEVICE))
+
+    ws = [w_eff[i].clone().requires_grad_(True) for i in range(n_mats)]
+    x_ref = x_pad.clone().requires_grad_(True)
+    y_ref = torch_reference(x_ref, ws, act, out_act)
+    assert max_norm_rel(y.detach().float().cpu().numpy(), y_ref[:, :n_out].detach().numpy()) <= 1e-2
+    y_ref[:, :n_out].backward(g.float())
+
+    # parameter gradients arrive in the parameter (packed) layout and in the parameter dtype
+    assert net.params.grad is not None and net.params.grad.shape == net.params.shape and net.params.grad.dtype == torch.float32
+    dW = unpack(net.params.grad.cpu().numpy().reshape(-1), n_mats, width)
+    assert x_dev.grad is not None and x_dev.grad.shape == (batch, n_in)
+    dx = x_dev.grad.float().cpu().numpy()
+
+    # (1) against the oracle, which rounds where the kernels round: it gets the loss-scaled dL/dy the module hands to
+    # the kernels, its results are divided by the loss scale as the module does
+    g_or = np.zeros((n_rows, width), np.float32)
+    g_or[:batch, :n_out] = (g * net.loss_scale).float().numpy()
+    _, dW_or, dX_or = oracle.mlp_backward_T(DT[dtype], width, n_mats, act, out_act, w_eff.numpy(), interm, g_or)
+    dW_or = dW_or.transpose(0, 2, 1) / net.loss_scale       # [out][in] -> [in][out]
+    dX_or = dX_or[:batch, :n_in] / net.loss_scale
+    assert_propagated(dW, dW_or, DT[dtype], "dW vs oracle", scale=float(np.abs(dW_or).max()))
+    assert_propagated(dx, dX_or, DT[dtype], "dL/dx vs oracle", scale=float(np.abs(dX_or).max()))
+
+    # (2) against fp32 autograd, as the reference's Python tests compare (test_compare_torch_dpcpp.py:185-242). The fp32
+    # chain does not round between layers, so a pre-activation within rounding distance of zero can get the other ReLU
+    # mask and move single gradient entries by one sample's worth (a tenth of the largest entry at batch 40); the
+    # check is therefore on the whole gradient: relative error in the Frobenius norm, 4e-2 for fp16 and 1e-1 for bf16
+    # (8 significant bits at each of the roundings on the way; measured 2.5e-2 and 6.5e-2 for dL/dx through five ReLU
+    # layers, where a flipped mask is not averaged over the batch). A wrong layout or scale gives an error of order 1.
+    dW_ref = np.stack([wi.grad.numpy() for wi in ws])
+    dx_ref = x_ref.grad[:, :n_in].numpy()
+    bar = 4e-2 if dtype == torch.float16 else 1e-1
+    for got, ref, what in ((dW, dW_ref, "dW"), (dx, dx_ref, "dL/dx")):
+        err = np.linalg.norm((got - ref).ravel()) / np.linalg.norm(ref.ravel())
+        assert err <= bar, f"{what}: relative Frobenius error {err:g} vs fp32 autograd"
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_set_params_constant(tcnn, dtype):
+    """test_set_param.py:24-70 of the reference."""
+    width = 16
+    net = tcnn.Network(16, 16, net_config(width, 3, "None", "None"), dtype=dtype)
+    x = (torch.ones(8, width) * 0.1).to(DEVICE, dtype=dtype)
+    param_vals = 0.123 * torch.ones(width * width * 4, 1, dtype=dtype).to(DEVICE)
+    net.set_params(param_vals)
+    assert torch.isclose(param_vals, net.params.to(dtype)).all()
+    assert torch.isclose(param_vals, net.params.data.to(dtype)).all()
+    y = net(x)
+    assert torch.isfinite(y).all()
+    # closed form: every layer multiplies by 16 * w (activation None)
+    w = float(torch.tensor(0.123, dtype=dtype))
+    expect = 0.1 * (16 * w) ** 4
+    assert torch.allclose(y.float(), torch.full_like(y.float(), expect), rtol=2e-2)
+
+
+@pytest.mark.parametrize("n_neurons", [16, 32, 64, 128])
+@pytest.mark.parametrize("n_hidden_layers", [1, 2, 4])
+def test_padding_weights_are_zero(tcnn, n_neurons, n_hidden_layers):
+    """test_padding_bias.py:176-213 of the reference: freshly initialised weights that only see padding are zero."""
+    n_in, n_out = 3, 5
+    net = tcnn.Network(n_in, n_out, net_config(n_neurons, n_hidden_layers, "none", "none"))
+    mats = unpack(net.get_params().float().cpu().numpy().reshape(-1), n_hidden_layers + 1, n_neurons)
+    assert np.all(mats[0][16:, :] == 0)       # use_bias=True: the input is padded with ones up to 16, zeros beyond
+    assert np.any(mats[0][:16, :] != 0)
+    assert np.all(mats[-1][:, n_out:] == 0)
+    assert np.any(mats[-1][:, :n_out] != 0)
+    # Xavier bound of the reference: +-sqrt(6 / (16 + width)) for the first and the last matrix, +-sqrt(6 / (2 width)) between
+    assert np.abs(mats[0]).max() <= (6.0 / (16 + n_neurons)) ** 0.5 * 1.01
+    for m in mats[1:-1]:
+        assert np.abs(m).max() <= (6.0 / (2 * n_neurons)) ** 0.5 * 1.01
+    # padded outputs of a network without output activation are exactly zero, whatever the input
+    x = torch.rand(24, n_in, device=DEVICE)
+    y_full = net.tnn_module.inference(torch.nn.functional.pad(x, [0, n_neurons - n_in], value=1.0).to(torch.float16).contiguous())
+    assert y_full.shape == (24, n_neurons) and torch.all(y_full[:, n_out:] == 0)
+
+
+def test_network_errors(tcnn):
+    with pytest.raises(RuntimeError, match="m_activation must be"):
+        tcnn.Network(16, 16, net_config(16, 2, "tanh", "none"))
+    with pytest.raises(NotImplementedError):
+        tcnn.Network(16, 16, net_config(16, 2, "swish", "none"))
+    with pytest.raises(AssertionError):
+        tcnn.Network(16, 16, net_config(16, 2), dtype=torch.float32)
+    with pytest.raises(RuntimeError, match="Unsupported width"):
+        tcnn.Network(16, 16, net_config(48, 2))
+    with pytest.raises(RuntimeError, match="not supported"):
+        tcnn.Network(65, 16, net_config(64, 2))
+    net = tcnn.Network(16, 16, net_config(16, 2))
+    with pytest.raises(RuntimeError, match="does not match"):
+        net.set_params(torch.zeros(5, device=DEVICE))
+    with pytest.raises((RuntimeError, ValueError), match="divisible by 8"):
+        net.tnn_module.inference(torch.zeros(7, 16, device=DEVICE, dtype=torch.float16))
+    with pytest.raises(RuntimeError, match="must be a GPU tensor"):
+        net.tnn_module.inference(torch.zeros(8, 16, dtype=torch.float16))
+    with pytest.raises(RuntimeError, match="takes no input_from_fwd"):
+        net.tnn_module.bwd_with_encoding_grad(torch.zeros(8, 16, device=DEVICE, dtype=torch.float16),
+                                              torch.zeros(8, 16, device=DEVICE, dtype=torch.float16), False, False)
+    # empty batch keeps its shape
+    y = net(torch.zeros(0, 16, device=DEVICE))
+    assert y.shape == (0, 16)
+    tcnn.free_temporary_memory()
+
+
+GRID_2D = {"otype": "HashGrid", "type": "Hash", "n_levels": 16, "n_features_per_level": 2, "log2_hashmap_size": 15,
+           "base_resolution": 16, "per_level_scale": 1.5}
+GRID_3D = {"otype": "HashGrid", "n_levels": 8, "n_features_per_level": 4, "log2_hashmap_size": 12, "base_resolution": 4,
+           "per_level_scale": 2.0, "interpolation": "Linear", "hash": "CoherentPrime"}
+
+
+def oracle_cfg(cfg, n_dims):
+    return {"n_dims": n_dims, "n_levels": cfg["n_levels"], "n_features_per_level": cfg["n_features_per_level"],
+            "log2_hashmap_size": cfg["log2_hashmap_size"], "base_resolution": cfg["base_resolution"],
+            "per_level_scale": cfg["per_level_scale"], "grid_type": cfg.get("type", "Hash"),
+            "hash": cfg.get("hash", "CoherentPrime"), "interpolation": cfg.get("interpolation", "Linear")}
+
+
+@pytest.mark.parametrize("cfg,n_dims,padded,batch", [(GRID_2D, 2, None, 1000), (GRID_2D, 2, 64, 256), (GRID_3D, 3, 64, 777)])
+def test_encoding_forward_and_gradients(tcnn, oracle, cfg, n_dims, padded, batch):
+    enc = tcnn.Encoding(n_dims, dict(cfg), n_output_dims=padded)
+    n_feat = cfg["n_levels"] * cfg["n_features_per_level"]
+    width = padded if padded is not None else n_feat
+    assert enc.n_output_dims == width
+    assert enc.params.dtype == torch.float32 and enc.params.requires_grad
+    init = enc.params.detach().cpu().numpy()
+    assert np.abs(init).max() <= 1e-4 and abs(init.mean()) < 1e-5 and init.std() > 3e-5   # uniform in +-1e-4
+
+    torch.manual_seed(3)
+    table = (torch.rand(enc.params.numel(), device=DEVICE) * 2 - 1)
+    enc.set_params(table)
+    np.testing.assert_array_equal(enc.get_params().cpu().numpy().reshape(-1), table.cpu().numpy())
+    np.testing.assert_array_equal(enc.params.detach().cpu().numpy().reshape(-1), table.cpu().numpy())
+
+    x = torch.rand(batch, n_dims)
+    x[0] = 0.0
+    x[1] = 1.0
+    y = enc(x.to(DEVICE))
+    assert y.shape == (batch, width) and y.dtype == torch.float32
+    ocfg = oracle_cfg(cfg, n_dims)
+    y_ref = oracle.grid_forward(ocfg, table.cpu().numpy(), x.numpy(), width)
+    np.testing.assert_allclose(y.detach().cpu().numpy(), y_ref, rtol=0, atol=2e-6)
+    if width > n_feat:
+        assert torch.all(y[:, n_feat:] == 0)
+
+    g = torch.rand(batch, width) * 2 - 1
+    y.backward(g.to(DEVICE))
+    grad = enc.params.grad.cpu().numpy().reshape(-1)
+    grad_ref = oracle.grid_backward(ocfg, x.numpy(), g.numpy(), table.numel())
+    assert max_norm_rel(grad, grad_ref) <= 1e-5
+
+
+def test_encoding_errors(tcnn):
+    with pytest.raises((RuntimeError, ValueError), match="Unknown encoding type"):
+        tcnn.Encoding(2, {"otype": "Nope"})
+    with pytest.raises(AssertionError):
+        tcnn.Encoding(2, dict(GRID_2D), dtype=torch.float16)
+    with pytest.raises((RuntimeError, ValueError), match="2 or 3"):
+        tcnn.Encoding(4, dict(GRID_2D))
+    enc = tcnn.Encoding(2, dict(GRID_2D))
+    with pytest.raises(RuntimeError, match="incorrect dimensions"):
+        enc.tnn_module.fwd(torch.zeros(8, 3, device=DEVICE))
+    with pytest.raises(RuntimeError, match="needs input_from_fwd"):
+        enc.tnn_module.bwd_no_encoding_grad(torch.zeros(8, 32, device=DEVICE), False, False)
+    with pytest.raises((RuntimeError, ValueError), match="not packed"):
+        enc.tnn_module.bwd_with_encoding_grad(torch.zeros(8, 32, device=DEVICE), torch.zeros(8, 2, device=DEVICE), True, False)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_network_with_input_encoding_trains(tcnn, dtype):
+    """BASELINE-style pipeline (2-D hash grid -> 64-wide MLP, 3 outputs) learning a smooth image with torch.optim.Adam."""
+    torch.manual_seed(1)
+    model = tcnn.NetworkWithInputEncoding(2, 3, net_config(64, 2), dict(GRID_2D), dtype=dtype, use_bias=False)
+    assert model.params is model.network.params
+    assert model.encoding.n_output_dims == 64
+    opt = torch.optim.Adam(model.parameters(), lr=1e-2, betas=(0.9, 0.99), eps=1e-15)
+    assert sum(p.numel() for p in model.parameters()) == model.network.params.numel() + model.encoding.params.numel()
+
+    def target(xy):
+        return torch.stack([torch.sin(6 * xy[:, 0]) * 0.5 + 0.5, xy[:, 1], xy[:, 0] * xy[:, 1]], dim=1)
+
+    losses = []
+    for step in range(60):
+        xy = torch.rand(4096, 2, device=DEVICE)
+        out = model(xy)
+        assert out.shape == (4096, 3) and out.dtype == dtype
+        loss = ((out.float() - target(xy)) ** 2).mean()
+        opt.zero_grad()
+        loss.backward()
+        assert model.network.params.grad is not None and model.encoding.params.grad is not None
+        assert torch.isfinite(model.network.params.grad).all() and torch.isfinite(model.encoding.params.grad).all()
+        opt.step()
+        losses.append(float(loss.detach()))
+    assert losses[-1] < 0.25 * losses[0], losses[::10]
+
+    model.eval()
+    with torch.no_grad():
+        xy = torch.rand(1001, 2, device=DEVICE)
+        out = model(xy)
+    assert out.shape == (1001, 3)
+    assert float(((out.float() - target(xy)) ** 2).mean()) < 0.5 * losses[0]
+    with pytest.raises(RuntimeError, match="Not implemented"):
+        model.get_params()

@@ -334,15 +334,15 @@ static int launch_grid_forward_o(const GridLevels &lv, const GridParams &gp, con
     const unsigned blocks = (unsigned)((M + kGridThreads - 1) / kGridThreads);
     switch (out_dtype) {
     case TNN_FP32:
-        hipLaunchKernelGGL((grid_forward_kernel<D, F, P, float>), dim3(blocks), dim3(kGridThreads), 0, s, lv, gp, x, (const P *)table,
+        TNN_LAUNCH((grid_forward_kernel<D, F, P, float>), dim3(blocks), dim3(kGridThreads), 0, s, lv, gp, x, (const P *)table,
                            (float *)out, (long long)M);
         break;
     case TNN_BF16:
-        hipLaunchKernelGGL((grid_forward_kernel<D, F, P, bf16_t>), dim3(blocks), dim3(kGridThreads), 0, s, lv, gp, x, (const P *)table,
+        TNN_LAUNCH((grid_forward_kernel<D, F, P, bf16_t>), dim3(blocks), dim3(kGridThreads), 0, s, lv, gp, x, (const P *)table,
                            (bf16_t *)out, (long long)M);
         break;
     case TNN_FP16:
-        hipLaunchKernelGGL((grid_forward_kernel<D, F, P, fp16_t>), dim3(blocks), dim3(kGridThreads), 0, s, lv, gp, x, (const P *)table,
+        TNN_LAUNCH((grid_forward_kernel<D, F, P, fp16_t>), dim3(blocks), dim3(kGridThreads), 0, s, lv, gp, x, (const P *)table,
                            (fp16_t *)out, (long long)M);
         break;
     default: return fail(TNN_ERR_UNSUPPORTED, "out_dtype %d", out_dtype);
@@ -363,15 +363,15 @@ static int launch_grid_backward_g(const GridLevels &lv, const GridParams &gp, co
     const dim3 grid((unsigned)((M + kGridThreads - 1) / kGridThreads), gp.n_levels);
     switch (dy_dtype) {
     case TNN_FP32:
-        hipLaunchKernelGGL((grid_backward_kernel<D, F, float>), grid, dim3(kGridThreads), 0, s, lv, gp, x, (const float *)dLdy, grad,
+        TNN_LAUNCH((grid_backward_kernel<D, F, float>), grid, dim3(kGridThreads), 0, s, lv, gp, x, (const float *)dLdy, grad,
                            (long long)M);
         break;
     case TNN_BF16:
-        hipLaunchKernelGGL((grid_backward_kernel<D, F, bf16_t>), grid, dim3(kGridThreads), 0, s, lv, gp, x, (const bf16_t *)dLdy, grad,
+        TNN_LAUNCH((grid_backward_kernel<D, F, bf16_t>), grid, dim3(kGridThreads), 0, s, lv, gp, x, (const bf16_t *)dLdy, grad,
                            (long long)M);
         break;
     case TNN_FP16:
-        hipLaunchKernelGGL((grid_backward_kernel<D, F, fp16_t>), grid, dim3(kGridThreads), 0, s, lv, gp, x, (const fp16_t *)dLdy, grad,
+        TNN_LAUNCH((grid_backward_kernel<D, F, fp16_t>), grid, dim3(kGridThreads), 0, s, lv, gp, x, (const fp16_t *)dLdy, grad,
                            (long long)M);
         break;
     default: return fail(TNN_ERR_UNSUPPORTED, "dy_dtype %d", dy_dtype);
@@ -505,7 +505,7 @@ TNN_API int tnn_grid_backward(const tnn_grid_desc *desc, const float *d_x, const
         size_t blocks = (n4 + 255) / 256;
         if (blocks > 4096) blocks = 4096;
         if (blocks < 4) blocks = 4;
-        hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)blocks), dim3(256), 0, s, (float4 *)d_grad_table, n4, d_grad_table + n4 * 4, n_tail);
+        TNN_LAUNCH(fill_zero_kernel, dim3((unsigned)blocks), dim3(256), 0, s, (float4 *)d_grad_table, n4, d_grad_table + n4 * 4, n_tail);
         if ((rc = check_launch("fill_zero_kernel"))) return rc;
     }
     TNN_DISPATCH_DF(desc, rc = (launch_grid_backward_g<D_, F_>(lv, gp, d_x, d_dLdy, dy_dtype, d_grad_table, M, s)));
@@ -520,8 +520,8 @@ TNN_API int tnn_grid_indices(const tnn_grid_desc *desc, const float *d_x, uint32
     if (!d_x || !d_indices) return fail(TNN_ERR_INVALID_ARGUMENT, "NULL pointer argument");
     const unsigned blocks = (unsigned)((M + kGridThreads - 1) / kGridThreads);
     if (desc->n_dims == 2)
-        hipLaunchKernelGGL((grid_indices_kernel<2>), dim3(blocks), dim3(kGridThreads), 0, as_stream(stream), lv, gp, d_x, d_indices, (long long)M);
+        TNN_LAUNCH((grid_indices_kernel<2>), dim3(blocks), dim3(kGridThreads), 0, as_stream(stream), lv, gp, d_x, d_indices, (long long)M);
     else
-        hipLaunchKernelGGL((grid_indices_kernel<3>), dim3(blocks), dim3(kGridThreads), 0, as_stream(stream), lv, gp, d_x, d_indices, (long long)M);
+        TNN_LAUNCH((grid_indices_kernel<3>), dim3(blocks), dim3(kGridThreads), 0, as_stream(stream), lv, gp, d_x, d_indices, (long long)M);
     return check_launch("grid_indices_kernel");
 }

@@ -66,10 +66,10 @@ static int launch_permute(int dtype, int W, int n_mats, const void *src, void *d
     if (src == dst) return fail(TNN_ERR_INVALID_ARGUMENT, "in-place permutation is not supported");
     const int total = W * W * n_mats;
     if (dtype == TNN_FP32)
-        hipLaunchKernelGGL((permute_kernel<float>), dim3((total + 255) / 256), dim3(256), 0, s, (const float *)src, (float *)dst,
+        TNN_LAUNCH((permute_kernel<float>), dim3((total + 255) / 256), dim3(256), 0, s, (const float *)src, (float *)dst,
                            W, n_mats, op);
     else
-        hipLaunchKernelGGL((permute_kernel<uint16_t>), dim3((total + 255) / 256), dim3(256), 0, s, (const uint16_t *)src,
+        TNN_LAUNCH((permute_kernel<uint16_t>), dim3((total + 255) / 256), dim3(256), 0, s, (const uint16_t *)src,
                            (uint16_t *)dst, W, n_mats, op);
     return check_launch("permute_kernel");
 }
@@ -202,7 +202,7 @@ TNN_API int tnn_zero_weights_padding(const tnn_mlp_desc *desc, void *d_packed, i
         one_padded = (unpadded_input_width / 16 + 1) * 16;
     if (one_padded > W) return fail(TNN_ERR_INVALID_ARGUMENT, "one_padded_input_width > padded_input_width, the input width is too small.");
     const int n_mats = desc->n_hidden_layers + 1;
-    hipLaunchKernelGGL((zero_padding_kernel<uint16_t>), dim3((W * W + 255) / 256), dim3(256), 0, as_stream(stream),
+    TNN_LAUNCH((zero_padding_kernel<uint16_t>), dim3((W * W + 255) / 256), dim3(256), 0, as_stream(stream),
                        (uint16_t *)d_packed, W, n_mats, one_padded, unpadded_output_width);
     return check_launch("zero_padding_kernel");
 }
@@ -217,10 +217,10 @@ TNN_API int tnn_l2_loss(int dtype, const void *d_predictions, const float *d_tar
     const float inv_n = 1.0f / (float)n_elements;
     const unsigned blocks = (unsigned)((n_elements + 255) / 256);
     if (dtype == TNN_BF16)
-        hipLaunchKernelGGL((l2_loss_kernel<bf16_t>), dim3(blocks), dim3(256), 0, as_stream(stream), (const bf16_t *)d_predictions,
+        TNN_LAUNCH((l2_loss_kernel<bf16_t>), dim3(blocks), dim3(256), 0, as_stream(stream), (const bf16_t *)d_predictions,
                            d_targets, n_elements, inv_n, loss_scale, d_values, (bf16_t *)d_grads);
     else
-        hipLaunchKernelGGL((l2_loss_kernel<fp16_t>), dim3(blocks), dim3(256), 0, as_stream(stream), (const fp16_t *)d_predictions,
+        TNN_LAUNCH((l2_loss_kernel<fp16_t>), dim3(blocks), dim3(256), 0, as_stream(stream), (const fp16_t *)d_predictions,
                            d_targets, n_elements, inv_n, loss_scale, d_values, (fp16_t *)d_grads);
     return check_launch("l2_loss_kernel");
 }
@@ -230,13 +230,13 @@ static int launch_adam(float *p, float *m, float *v, const void *g, float gs, si
                        float b1, float b2, float eps, void *pT, int pT_dtype, hipStream_t s) {
     const unsigned blocks = (unsigned)((n + 255) / 256);
     if (pT && pT_dtype == TNN_BF16)
-        hipLaunchKernelGGL((adam_kernel<G, bf16_t>), dim3(blocks), dim3(256), 0, s, p, m, v, (const G *)g, gs, n, step_size,
+        TNN_LAUNCH((adam_kernel<G, bf16_t>), dim3(blocks), dim3(256), 0, s, p, m, v, (const G *)g, gs, n, step_size,
                            bc2_sqrt, b1, b2, eps, (bf16_t *)pT);
     else if (pT && pT_dtype == TNN_FP16)
-        hipLaunchKernelGGL((adam_kernel<G, fp16_t>), dim3(blocks), dim3(256), 0, s, p, m, v, (const G *)g, gs, n, step_size,
+        TNN_LAUNCH((adam_kernel<G, fp16_t>), dim3(blocks), dim3(256), 0, s, p, m, v, (const G *)g, gs, n, step_size,
                            bc2_sqrt, b1, b2, eps, (fp16_t *)pT);
     else
-        hipLaunchKernelGGL((adam_kernel<G, float>), dim3(blocks), dim3(256), 0, s, p, m, v, (const G *)g, gs, n, step_size,
+        TNN_LAUNCH((adam_kernel<G, float>), dim3(blocks), dim3(256), 0, s, p, m, v, (const G *)g, gs, n, step_size,
                            bc2_sqrt, b1, b2, eps, (float *)pT);
     return check_launch("adam_kernel");
 }
@@ -283,11 +283,11 @@ TNN_API int tnn_mlp_adam_update(const tnn_mlp_desc *desc, float *d_master_packed
     const int total = W * W * n_mats;
     hipStream_t s = as_stream(stream);
     if (desc->dtype == TNN_BF16)
-        hipLaunchKernelGGL((mlp_adam_update_kernel<bf16_t>), dim3((total + 255) / 256), dim3(256), 0, s, d_master_packed, d_m, d_v, d_dW_raw,
+        TNN_LAUNCH((mlp_adam_update_kernel<bf16_t>), dim3((total + 255) / 256), dim3(256), 0, s, d_master_packed, d_m, d_v, d_dW_raw,
                            grad_scale, W, n_mats, step_size, bc2_sqrt, beta1, beta2, eps, (bf16_t *)d_packed_T, (bf16_t *)d_prepared_fwd,
                            (bf16_t *)d_prepared_bwd);
     else
-        hipLaunchKernelGGL((mlp_adam_update_kernel<fp16_t>), dim3((total + 255) / 256), dim3(256), 0, s, d_master_packed, d_m, d_v, d_dW_raw,
+        TNN_LAUNCH((mlp_adam_update_kernel<fp16_t>), dim3((total + 255) / 256), dim3(256), 0, s, d_master_packed, d_m, d_v, d_dW_raw,
                            grad_scale, W, n_mats, step_size, bc2_sqrt, beta1, beta2, eps, (fp16_t *)d_packed_T, (fp16_t *)d_prepared_fwd,
                            (fp16_t *)d_prepared_bwd);
     return check_launch("mlp_adam_update_kernel");
@@ -300,9 +300,9 @@ TNN_API int tnn_fill(int dtype, void *d_ptr, size_t n, float value, tnn_stream_t
     if (blocks > 8192) blocks = 8192;
     hipStream_t s = as_stream(stream);
     switch (dtype) {
-    case TNN_BF16: hipLaunchKernelGGL((fill_kernel<bf16_t>), dim3((unsigned)blocks), dim3(256), 0, s, (bf16_t *)d_ptr, n, (bf16_t)value); break;
-    case TNN_FP16: hipLaunchKernelGGL((fill_kernel<fp16_t>), dim3((unsigned)blocks), dim3(256), 0, s, (fp16_t *)d_ptr, n, (fp16_t)value); break;
-    case TNN_FP32: hipLaunchKernelGGL((fill_kernel<float>), dim3((unsigned)blocks), dim3(256), 0, s, (float *)d_ptr, n, value); break;
+    case TNN_BF16: TNN_LAUNCH((fill_kernel<bf16_t>), dim3((unsigned)blocks), dim3(256), 0, s, (bf16_t *)d_ptr, n, (bf16_t)value); break;
+    case TNN_FP16: TNN_LAUNCH((fill_kernel<fp16_t>), dim3((unsigned)blocks), dim3(256), 0, s, (fp16_t *)d_ptr, n, (fp16_t)value); break;
+    case TNN_FP32: TNN_LAUNCH((fill_kernel<float>), dim3((unsigned)blocks), dim3(256), 0, s, (float *)d_ptr, n, value); break;
     default: return fail(TNN_ERR_UNSUPPORTED, "dtype %d", dtype);
     }
     return check_launch("fill_kernel");
@@ -312,9 +312,9 @@ template <typename D> static int launch_cast(D *d, int src_dtype, const void *sr
     size_t blocks = (n + 255) / 256;
     if (blocks > 8192) blocks = 8192;
     switch (src_dtype) {
-    case TNN_BF16: hipLaunchKernelGGL((cast_kernel<D, bf16_t>), dim3((unsigned)blocks), dim3(256), 0, s, d, (const bf16_t *)src, n); break;
-    case TNN_FP16: hipLaunchKernelGGL((cast_kernel<D, fp16_t>), dim3((unsigned)blocks), dim3(256), 0, s, d, (const fp16_t *)src, n); break;
-    case TNN_FP32: hipLaunchKernelGGL((cast_kernel<D, float>), dim3((unsigned)blocks), dim3(256), 0, s, d, (const float *)src, n); break;
+    case TNN_BF16: TNN_LAUNCH((cast_kernel<D, bf16_t>), dim3((unsigned)blocks), dim3(256), 0, s, d, (const bf16_t *)src, n); break;
+    case TNN_FP16: TNN_LAUNCH((cast_kernel<D, fp16_t>), dim3((unsigned)blocks), dim3(256), 0, s, d, (const fp16_t *)src, n); break;
+    case TNN_FP32: TNN_LAUNCH((cast_kernel<D, float>), dim3((unsigned)blocks), dim3(256), 0, s, d, (const float *)src, n); break;
     default: return fail(TNN_ERR_UNSUPPORTED, "src dtype %d", src_dtype);
     }
     return check_launch("cast_kernel");

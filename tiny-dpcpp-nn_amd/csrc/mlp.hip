@@ -382,11 +382,11 @@ static int launch_forward_v(const tnn_mlp_desc *d, const void *wprep, const void
             hipFuncSetAttribute(reinterpret_cast<const void *>(k), hipFuncAttributeMaxDynamicSharedMemorySize,
                                 (int)wbytes) != hipSuccess)
             return fail(TNN_ERR_HIP, "cannot reserve %zu bytes of LDS", wbytes);
-        hipLaunchKernelGGL(k, dim3((unsigned)blocks), dim3(THREADS), wbytes, s, (const vec8 *)wprep, (const T *)x,
+        TNN_LAUNCH(k, dim3((unsigned)blocks), dim3(THREADS), wbytes, s, (const vec8 *)wprep, (const T *)x,
                            (T *)out, n_mats, d->output_activation, (long long)M);
     } else {
         auto k = mlp_forward_kernel<T, W, ACT, STORE_INTERM, false, THREADS, PREFETCH>;
-        hipLaunchKernelGGL(k, dim3((unsigned)blocks), dim3(THREADS), 0, s, (const vec8 *)wprep, (const T *)x, (T *)out,
+        TNN_LAUNCH(k, dim3((unsigned)blocks), dim3(THREADS), 0, s, (const vec8 *)wprep, (const T *)x, (T *)out,
                            n_mats, d->output_activation, (long long)M);
     }
     return check_launch("mlp_forward_kernel");
@@ -430,12 +430,12 @@ static int launch_backward(const tnn_mlp_desc *d, const void *wprep_bwd, const v
                                 (int)wbytes) != hipSuccess)
             return fail(TNN_ERR_HIP, "cannot reserve %zu bytes of LDS", wbytes);
         const long long blocks = stream_grid(reinterpret_cast<const void *>(k), wbytes, M, di.n_cu);
-        hipLaunchKernelGGL(k, dim3((unsigned)blocks), dim3(kFwdThreads), wbytes, s, (const vec8 *)wprep_bwd,
+        TNN_LAUNCH(k, dim3((unsigned)blocks), dim3(kFwdThreads), wbytes, s, (const vec8 *)wprep_bwd,
                            (const T *)dLdy, (const T *)interm_fwd, (T *)interm_bwd, (T *)dLdx, n_mats, d->activation,
                            d->output_activation, (long long)M);
     } else {
         const long long blocks = stream_grid(reinterpret_cast<const void *>(mlp_backward_kernel<T, W, false>), 0, M, di.n_cu);
-        hipLaunchKernelGGL((mlp_backward_kernel<T, W, false>), dim3((unsigned)blocks), dim3(kFwdThreads), 0, s,
+        TNN_LAUNCH((mlp_backward_kernel<T, W, false>), dim3((unsigned)blocks), dim3(kFwdThreads), 0, s,
                            (const vec8 *)wprep_bwd, (const T *)dLdy, (const T *)interm_fwd, (T *)interm_bwd, (T *)dLdx,
                            n_mats, d->activation, d->output_activation, (long long)M);
     }
@@ -470,12 +470,12 @@ static int launch_dw(const tnn_mlp_desc *d, const void *interm_bwd, const void *
                      size_t M, float *partials, hipStream_t s) {
     const int n_mats = d->n_hidden_layers + 1;
     const DwPlan p = dw_plan(d, M);
-    hipLaunchKernelGGL((mlp_dw_partial_kernel<T, W>), dim3((unsigned)p.n_chunks, (unsigned)n_mats), dim3(kDwThreads), 0, s,
+    TNN_LAUNCH((mlp_dw_partial_kernel<T, W>), dim3((unsigned)p.n_chunks, (unsigned)n_mats), dim3(kDwThreads), 0, s,
                        (const T *)interm_bwd, (const T *)interm_fwd, partials, n_mats, (long long)M, p.rows_per_chunk);
     int rc = check_launch("mlp_dw_partial_kernel");
     if (rc) return rc;
     const int n_elems = n_mats * W * W;
-    hipLaunchKernelGGL((dw_reduce_kernel<T>), dim3((n_elems + 255) / 256), dim3(256), 0, s, partials,
+    TNN_LAUNCH((dw_reduce_kernel<T>), dim3((n_elems + 255) / 256), dim3(256), 0, s, partials,
                        (int)(p.n_chunks * p.partials_per_chunk), n_elems, dW_is_fp32 ? (T *)nullptr : (T *)dW,
                        dW_is_fp32 ? (float *)dW : (float *)nullptr);
     return check_launch("dw_reduce_kernel");
@@ -526,18 +526,18 @@ TNN_API int tnn_mlp_prepare_weights(const tnn_mlp_desc *desc, const void *d_pack
     hipStream_t s = as_stream(stream);
     if (desc->dtype == TNN_BF16) {
         if (src_is_fp32)
-            hipLaunchKernelGGL((prepare_weights_kernel<bf16_t, float>), dim3(blocks), dim3(256), 0, s, (const float *)d_packed,
+            TNN_LAUNCH((prepare_weights_kernel<bf16_t, float>), dim3(blocks), dim3(256), 0, s, (const float *)d_packed,
                                (bf16_t *)d_prepared_fwd, (bf16_t *)d_prepared_bwd, desc->width, n_mats);
         else
-            hipLaunchKernelGGL((prepare_weights_kernel<bf16_t, bf16_t>), dim3(blocks), dim3(256), 0, s,
+            TNN_LAUNCH((prepare_weights_kernel<bf16_t, bf16_t>), dim3(blocks), dim3(256), 0, s,
                                (const bf16_t *)d_packed, (bf16_t *)d_prepared_fwd, (bf16_t *)d_prepared_bwd, desc->width,
                                n_mats);
     } else {
         if (src_is_fp32)
-            hipLaunchKernelGGL((prepare_weights_kernel<fp16_t, float>), dim3(blocks), dim3(256), 0, s, (const float *)d_packed,
+            TNN_LAUNCH((prepare_weights_kernel<fp16_t, float>), dim3(blocks), dim3(256), 0, s, (const float *)d_packed,
                                (fp16_t *)d_prepared_fwd, (fp16_t *)d_prepared_bwd, desc->width, n_mats);
         else
-            hipLaunchKernelGGL((prepare_weights_kernel<fp16_t, fp16_t>), dim3(blocks), dim3(256), 0, s,
+            TNN_LAUNCH((prepare_weights_kernel<fp16_t, fp16_t>), dim3(blocks), dim3(256), 0, s,
                                (const fp16_t *)d_packed, (fp16_t *)d_prepared_fwd, (fp16_t *)d_prepared_bwd, desc->width,
                                n_mats);
     }

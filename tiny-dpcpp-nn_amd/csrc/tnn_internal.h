@@ -22,6 +22,14 @@ inline hipStream_t as_stream(tnn_stream_t s) { return reinterpret_cast<hipStream
 // Reports a failed launch as TNN_ERR_HIP. Does not synchronize.
 int check_launch(const char *what);
 
+// Every kernel goes out through this: an error that an earlier, unrelated runtime call of this thread left
+// behind (a failed allocation of the caller, say) is dropped first, so that check_launch reports this launch only.
+#define TNN_LAUNCH(...)                                                                                                \
+    do {                                                                                                               \
+        (void)hipGetLastError();                                                                                       \
+        hipLaunchKernelGGL(__VA_ARGS__);                                                                               \
+    } while (0)
+
 inline bool valid_width(int w) { return w == 16 || w == 32 || w == 64 || w == 128; }
 inline bool valid_act(int a) { return a == TNN_ACT_NONE || a == TNN_ACT_RELU || a == TNN_ACT_SIGMOID; }
 int check_mlp_desc(const tnn_mlp_desc *d);

@@ -78,15 +78,15 @@ TNN_API int tnn_mlp_train_step_l2(const tnn_mlp_desc *desc, const void *d_prepar
     const void *y = static_cast<const char *>(interm_fwd) + (size_t)n_mats * mat;
     if (d_y && hipMemcpyAsync(d_y, y, mat, hipMemcpyDeviceToDevice, s) != hipSuccess) return fail(TNN_ERR_HIP, "copy of the network output failed");
     const size_t n = M * W;
-    if (d_loss_sum) hipLaunchKernelGGL(zero_scalar_kernel, dim3(1), dim3(1), 0, s, d_loss_sum);
+    if (d_loss_sum) TNN_LAUNCH(zero_scalar_kernel, dim3(1), dim3(1), 0, s, d_loss_sum);
     size_t blocks = (n + 256 * 8 - 1) / (256 * 8);
     if (blocks > 2048) blocks = 2048;
     const float inv_n = 1.0f / (float)n;
     if (desc->dtype == TNN_BF16)
-        hipLaunchKernelGGL((l2_loss_sum_kernel<bf16_t>), dim3((unsigned)blocks), dim3(256), 0, s, (const bf16_t *)y, d_targets, n, inv_n,
+        TNN_LAUNCH((l2_loss_sum_kernel<bf16_t>), dim3((unsigned)blocks), dim3(256), 0, s, (const bf16_t *)y, d_targets, n, inv_n,
                            loss_scale, d_loss_sum, (bf16_t *)dLdy);
     else
-        hipLaunchKernelGGL((l2_loss_sum_kernel<fp16_t>), dim3((unsigned)blocks), dim3(256), 0, s, (const fp16_t *)y, d_targets, n, inv_n,
+        TNN_LAUNCH((l2_loss_sum_kernel<fp16_t>), dim3((unsigned)blocks), dim3(256), 0, s, (const fp16_t *)y, d_targets, n, inv_n,
                            loss_scale, d_loss_sum, (fp16_t *)dLdy);
     if ((rc = check_launch("l2_loss_sum_kernel"))) return rc;
     return tnn_mlp_backward(desc, d_prepared_bwd, dLdy, interm_fwd, nullptr, d_dW, dW_is_fp32, d_dLdx, M, bwd_ws, bwd_ws_bytes, stream);

@@ -60,7 +60,9 @@ template <typename T> class DeviceMatricesView {
     uint32_t n_matrices() const { return n_matrices_; }
     size_t input_m() const { return input_m_; }
     size_t input_n() const { return input_n_; }
+    size_t middle_m() const { return middle_m_; }
     size_t middle_n() const { return middle_n_; }
+    size_t output_m() const { return output_m_; }
     size_t output_n() const { return output_n_; }
 
   private:

@@ -1,0 +1,385 @@
+// The tensor-level module interface that the Python bindings wrap. Mirrors include/tnn_api.h of the reference:
+// tnn::Module (:62-303), EncodingModule<T> (:306-474), NetworkModule<T, WIDTH> (:477-697). Tensors are
+// PyTorch-ROCm tensors on the GPU; the stream is torch's current HIP stream at construction (the reference takes
+// the current XPU stream's queue, :295-302). Results are handed back as fresh torch allocations (clones of the
+// module's grow-only workspaces), and every method blocks until its work is done, as in the reference.
+#pragma once
+
+#include <c10/hip/HIPStream.h>
+#include <torch/torch.h>
+
+#include <tuple>
+
+#include "SwiftNetMLP.h"
+#include "encoding_factory.h"
+#include "io.h"
+
+#define CHECK_GPU(x) TORCH_CHECK(x.device().is_cuda(), #x " must be a GPU tensor")
+#define CHECK_CONTIGUOUS(x) TORCH_CHECK(x.is_contiguous(), #x " must be contiguous")
+#define CHECK_INPUT(x)                                                                                                 \
+    CHECK_GPU(x);                                                                                                      \
+    CHECK_CONTIGUOUS(x)
+
+namespace tnn {
+
+using fp16 = tnn::half;
+
+template <typename T> struct torch_type {};
+template <> struct torch_type<int> { static constexpr auto dtype = torch::kInt32; };
+template <> struct torch_type<double> { static constexpr auto dtype = torch::kFloat64; };
+template <> struct torch_type<float> { static constexpr auto dtype = torch::kFloat32; };
+template <> struct torch_type<fp16> { static constexpr auto dtype = c10::ScalarType::Half; };
+template <> struct torch_type<bf16> { static constexpr auto dtype = c10::ScalarType::BFloat16; };
+
+class Module {
+  public:
+    Module() : queue_(c10::hip::getCurrentHIPStream().stream()), device_index_(c10::hip::current_device()) {}
+    virtual ~Module() {}
+
+    virtual torch::Tensor initialize_params() = 0;
+    virtual torch::Tensor initialize_params(const torch::Tensor &tensor) = 0;
+    virtual void set_params(const torch::Tensor &tensor, bool weights_are_packed) = 0;
+    virtual torch::Tensor get_params() = 0;
+    virtual torch::Tensor forward_pass(const torch::Tensor &input_tensor) = 0;
+    virtual std::tuple<torch::Tensor, torch::Tensor> backward_pass(const torch::Tensor &input_tensor, const torch::Tensor &input_from_fwd,
+                                                                   bool pack_transpose_gradient, bool get_dl_dinput) = 0;
+    virtual std::tuple<torch::Tensor, torch::Tensor> backward_pass(const torch::Tensor &input_tensor, bool pack_transpose_gradient,
+                                                                   bool get_dl_dinput) = 0;
+    virtual torch::Tensor inference(const torch::Tensor &input_tensor) = 0;
+    virtual size_t n_params() = 0;
+    virtual size_t n_output_dims() = 0;
+
+    tnn::queue &get_queue() { return queue_; }
+
+    template <typename T> static std::vector<T> convertTensorToVector(const torch::Tensor &tensor) {
+        const auto cpu = tensor.to(torch::kCPU).to(torch::kFloat32).contiguous();
+        const float *begin = cpu.data_ptr<float>();
+        std::vector<T> result;
+        result.reserve(cpu.numel());
+        for (int64_t i = 0; i < cpu.numel(); ++i) result.push_back(T(begin[i]));
+        return result;
+    }
+
+    template <typename T> torch::Tensor convertVectorToTensor(const std::vector<T> &v) const {
+        std::vector<float> f(v.begin(), v.end());
+        return torch::from_blob(f.data(), {(int64_t)f.size()}, torch::TensorOptions().dtype(torch::kFloat32)).clone().to(device());
+    }
+
+    /// Fresh tensor holding a copy of device memory owned by the module.
+    template <typename T> torch::Tensor fromDevice(T *ptr, std::initializer_list<int64_t> sizes) const {
+        return torch::from_blob(ptr, sizes, torch::TensorOptions().dtype(torch_type<T>::dtype).device(device())).clone();
+    }
+    template <typename T> torch::Tensor convertDeviceMatrixViewToTorchTensor(const DeviceMatrixView<T> &dm) const {
+        return fromDevice<T>(dm.GetPointer(), {(int64_t)dm.m(), (int64_t)dm.n()});
+    }
+    template <typename T> torch::Tensor convertDeviceMatrixToTorchTensor(DeviceMatrix<T> &dm) const {
+        return fromDevice<T>(dm.data(), {(int64_t)dm.rows(), (int64_t)dm.cols()});
+    }
+    template <typename T> torch::Tensor convertDeviceMatricesToTorchTensor(const DeviceMatrices<T> &dm) const {
+        return fromDevice<T>(dm.GetViews().GetMatrixPointer(0), {(int64_t)dm.nelements(), 1});
+    }
+
+  protected:
+    virtual void FreeWorkspace() = 0;
+    virtual void AllocateWorkspace(const size_t batch_size) = 0;
+    c10::Device device() const { return c10::Device(c10::DeviceType::CUDA, device_index_); }
+
+  private:
+    tnn::queue queue_;
+    c10::DeviceIndex device_index_;
+};
+
+/************************************************ENCODING MODULE */
+template <typename T> class EncodingModule : public Module {
+  public:
+    EncodingModule(std::string filename, std::optional<uint32_t> padded_output_width = std::nullopt)
+        : max_batch_size_(0), output_encoding_ptr_(nullptr) {
+        encoding_ = create_encoding<T>(io::loadJsonConfig(filename), this->get_queue(), padded_output_width);
+        initialize_ptr();
+    }
+
+    EncodingModule(const json &encoding_config, std::optional<uint32_t> padded_output_width = std::nullopt)
+        : max_batch_size_(0), output_encoding_ptr_(nullptr) {
+        encoding_ = create_encoding<T>(io::validateAndCopyEncodingConfig(encoding_config), this->get_queue(), padded_output_width);
+        initialize_ptr();
+    }
+
+    ~EncodingModule() { this->FreeWorkspace(); }
+
+    torch::Tensor forward_pass(const torch::Tensor &input_tensor) override {
+        CHECK_INPUT(input_tensor);
+        TORCH_CHECK(input_tensor.scalar_type() == torch::kFloat32, "input_tensor must be float32");
+        const size_t batch_size = input_tensor.sizes()[0];
+        if (input_tensor.sizes().size() != 2 || input_tensor.sizes()[1] != encoding_->get_input_width())
+            throw std::runtime_error("Input tensor has incorrect dimensions");
+        const uint32_t out_w = encoding_->get_padded_output_width();
+        if (batch_size == 0) return torch::empty({0, (int64_t)out_w}, torch::TensorOptions().dtype(torch_type<T>::dtype).device(device()));
+
+        DeviceMatrixView<float> input_dmv(batch_size, encoding_->get_input_width(), encoding_->get_input_width(), input_tensor.data_ptr<float>());
+        this->AllocateWorkspace(batch_size);
+        DeviceMatrixView<T> output_encoding(batch_size, out_w, out_w, output_encoding_ptr_);
+        std::unique_ptr<Context> model_ctx = encoding_->forward_impl(input_dmv, &output_encoding);
+        this->get_queue().wait();
+        return fromDevice<T>(output_encoding.GetPointer(), {(int64_t)batch_size, (int64_t)out_w});
+    }
+
+    torch::Tensor inference(const torch::Tensor &input_tensor) override { return forward_pass(input_tensor); }
+
+    std::tuple<torch::Tensor, torch::Tensor> backward_pass(const torch::Tensor &, bool = false, bool = false) override {
+        throw std::runtime_error("backward_pass needs input_from_fwd");
+    }
+
+    std::tuple<torch::Tensor, torch::Tensor> backward_pass(const torch::Tensor &grad_output, const torch::Tensor &input_from_fwd,
+                                                           bool pack_transpose_gradient = false, bool get_dl_dinput = false) override {
+        if (encoding_->get_n_params() == 0) return {torch::Tensor(), torch::Tensor()};
+        CHECK_INPUT(grad_output);
+        CHECK_INPUT(input_from_fwd);
+        if (pack_transpose_gradient) throw std::invalid_argument("Encoding params are not packed");
+        if (get_dl_dinput) throw std::invalid_argument("Encoding get_dl_dinput not implemented");
+        TORCH_CHECK(grad_output.scalar_type() == torch_type<T>::dtype, "grad_output has the wrong dtype");
+        TORCH_CHECK(input_from_fwd.scalar_type() == torch::kFloat32, "input_from_fwd must be float32");
+
+        const int64_t batch_size = grad_output.sizes()[0];
+        const int64_t input_width = encoding_->get_input_width();
+        const auto input_sizes = input_from_fwd.sizes();
+        if (input_sizes.size() != 2 || input_sizes[0] != batch_size || input_sizes[1] != input_width)
+            throw std::runtime_error("Size mismatch for input_from_fwd: expected [" + std::to_string(batch_size) + ", " +
+                                     std::to_string(input_width) + "], but got [" + std::to_string(input_sizes[0]) + ", " +
+                                     std::to_string(input_sizes.size() > 1 ? input_sizes[1] : 0) + "]");
+        if (grad_output.sizes().size() != 2 || grad_output.sizes()[1] != encoding_->get_padded_output_width())
+            throw std::runtime_error("grad_output must be [batch, padded output width]");
+
+        const uint32_t out_w = encoding_->get_padded_output_width();
+        DeviceMatrixView<T> dL_doutput_dmv(batch_size, out_w, out_w, reinterpret_cast<T *>(grad_output.data_ptr()));
+        DeviceMatrixView<float> input_encoding_dmv(batch_size, input_width, input_width, input_from_fwd.data_ptr<float>());
+        auto gradients_view = gradients_->GetView();
+        Context ctx;
+        encoding_->backward_impl(ctx, input_encoding_dmv, dL_doutput_dmv, &gradients_view);
+        this->get_queue().wait();
+        return {torch::Tensor(), convertDeviceMatrixToTorchTensor(*gradients_)};
+    }
+
+    torch::Tensor initialize_params() override { return get_params(); }
+    torch::Tensor initialize_params(const torch::Tensor &tensor) override {
+        set_params(tensor, false);
+        return get_params();
+    }
+
+    void set_params(const torch::Tensor &params, bool weights_are_packed) override {
+        if (encoding_->get_params() == nullptr) throw std::runtime_error("no encoding params to set");
+        if (weights_are_packed) throw std::runtime_error("Packed weights are not supported in api set params");
+        CHECK_INPUT(params);
+        TORCH_CHECK((size_t)params.numel() == encoding_->get_n_params(), "params has ", params.numel(), " elements, the encoding has ",
+                    encoding_->get_n_params());
+        TORCH_CHECK(params.scalar_type() == torch_type<T>::dtype, "params has the wrong dtype");
+        encoding_->get_params()->copy_from_device(params.data_ptr<T>());
+    }
+
+    torch::Tensor get_params() override {
+        if (encoding_->get_params()) return convertDeviceMatrixToTorchTensor<T>(*encoding_->get_params());
+        return torch::empty({0});
+    }
+
+    size_t n_params() override { return encoding_->get_n_params(); }
+    size_t n_output_dims() override { return encoding_->get_padded_output_width(); }
+    std::vector<T> get_encoding_params() { return encoding_->get_params()->copy_to_host(); }
+    std::vector<T> get_encoding_grads() { return gradients_->copy_to_host(); }
+
+  protected:
+    void FreeWorkspace() override {
+        tnn::detail::device_free(output_encoding_ptr_);
+        output_encoding_ptr_ = nullptr;
+        max_batch_size_ = 0;
+    }
+
+    void AllocateWorkspace(const size_t batch_size) override {
+        if (batch_size > max_batch_size_) {
+            this->get_queue().wait();
+            this->FreeWorkspace();
+            output_encoding_ptr_ = tnn::detail::device_alloc<T>(batch_size * encoding_->get_padded_output_width());
+            max_batch_size_ = batch_size;
+        }
+    }
+
+  private:
+    void initialize_ptr() {
+        if (encoding_ && encoding_->get_n_params()) {
+            gradients_ = std::make_unique<DeviceMatrix<T>>(encoding_->get_n_params(), 1, this->get_queue());
+            gradients_->fill(0.0f).wait();
+        }
+    }
+
+    std::shared_ptr<Encoding<T>> encoding_;
+    std::unique_ptr<DeviceMatrix<T>> gradients_;
+    size_t max_batch_size_; // the workspace fits every batch size seen so far
+    T *output_encoding_ptr_;
+};
+
+/**************************************NETWORK MODULE */
+template <typename T, int WIDTH> class NetworkModule : public Module {
+  public:
+    NetworkModule(const int input_width, const int output_width, const int n_hidden_layers, const Activation activation,
+                  const Activation output_activation, bool use_bias)
+        : network_(this->get_queue(), input_width, output_width, n_hidden_layers, activation, output_activation,
+                   Network<T>::WeightInitMode::xavier_normal, use_bias),
+          net_gradients_(network_.get_n_hidden_layers() + 1, network_.get_network_width(), WIDTH, WIDTH, WIDTH, WIDTH,
+                         network_.get_output_width(), this->get_queue()),
+          max_batch_size_(0), interm_forw_ptr_(nullptr), interm_backw_ptr_(nullptr), dL_dinput_ptr_(nullptr) {
+        net_gradients_.fill(T(0.0f)).wait();
+    }
+
+    ~NetworkModule() { this->FreeWorkspace(); }
+
+    torch::Tensor inference(const torch::Tensor &input_tensor) override {
+        const size_t batch_size = CheckedBatch(input_tensor, network_.get_input_width());
+        const int64_t out_w = network_.get_output_width();
+        if (batch_size == 0) return torch::empty({0, out_w}, torch::TensorOptions().dtype(torch_type<T>::dtype).device(device()));
+        DeviceMatrixView<T> input_dm(batch_size, network_.get_input_width(), network_.get_input_width(),
+                                     reinterpret_cast<T *>(input_tensor.data_ptr()));
+        this->AllocateWorkspace(batch_size);
+        DeviceMatricesView<T> output_network(1, batch_size, network_.get_output_width(), 0, 0, 0, 0, interm_forw_ptr_);
+        network_.inference(input_dm, output_network, {});
+        this->get_queue().wait();
+        return fromDevice<T>(interm_forw_ptr_, {(int64_t)batch_size, out_w});
+    }
+
+    torch::Tensor forward_pass(const torch::Tensor &input_tensor) override {
+        const size_t batch_size = CheckedBatch(input_tensor, network_.get_input_width());
+        const int64_t out_w = network_.get_output_width();
+        if (batch_size == 0) return torch::empty({0, out_w}, torch::TensorOptions().dtype(torch_type<T>::dtype).device(device()));
+        DeviceMatrixView<T> input_dm(batch_size, network_.get_input_width(), network_.get_input_width(),
+                                     reinterpret_cast<T *>(input_tensor.data_ptr()));
+        this->AllocateWorkspace(batch_size);
+        DeviceMatricesView<T> output_network = ForwardViews(batch_size);
+        network_.forward_pass(input_dm, output_network, {});
+        this->get_queue().wait();
+        forward_batch_size_ = batch_size;
+        return fromDevice<T>(output_network.GetMatrixPointer(network_.get_n_hidden_layers() + 1), {(int64_t)batch_size, out_w});
+    }
+
+    std::tuple<torch::Tensor, torch::Tensor> backward_pass(const torch::Tensor &, const torch::Tensor &, bool, bool) override {
+        throw std::runtime_error("backward_pass of NetworkModule takes no input_from_fwd");
+    }
+
+    std::tuple<torch::Tensor, torch::Tensor> backward_pass(const torch::Tensor &grad_output, bool pack_transpose_gradient,
+                                                           bool get_dl_dinput) override {
+        CHECK_INPUT(grad_output);
+        TORCH_CHECK(grad_output.dim() == 2, "grad_output must have two dimensions");
+        TORCH_CHECK(grad_output.scalar_type() == torch_type<T>::dtype, "grad_output has the wrong dtype");
+        const size_t batch_size = grad_output.sizes()[0];
+        if (grad_output.size(1) != network_.get_output_width())
+            throw std::invalid_argument("grad_output.size(1): " + std::to_string(grad_output.size(1)) +
+                                        " is not equal to  get_padded_output_width" + std::to_string(network_.get_output_width()));
+        if (batch_size % 8 != 0) throw std::invalid_argument("Batch size is not divisible by 8.");
+        // The activations of the last forward_pass are the other operand; they live in the module's workspace.
+        if (batch_size == 0 || batch_size != forward_batch_size_)
+            throw std::invalid_argument("backward_pass: batch size " + std::to_string(batch_size) +
+                                        " does not match the last forward_pass (" + std::to_string(forward_batch_size_) + ")");
+
+        DeviceMatrixView<T> dL_doutput(batch_size, network_.get_output_width(), network_.get_output_width(),
+                                       reinterpret_cast<T *>(grad_output.data_ptr()));
+        DeviceMatricesView<T> interm_bwd(network_.get_n_hidden_layers() + 1, batch_size, network_.get_input_width(), batch_size,
+                                         network_.get_network_width(), batch_size, network_.get_output_width(), interm_backw_ptr_);
+        DeviceMatricesView<T> interm_fwd = ForwardViews(batch_size);
+        DeviceMatrixView<T> dL_dinput(batch_size, network_.get_input_width(), network_.get_input_width(), dL_dinput_ptr_);
+
+        network_.backward_pass(dL_doutput, net_gradients_.GetViews(), interm_bwd, interm_fwd, {}, get_dl_dinput ? &dL_dinput : nullptr);
+        this->get_queue().wait();
+
+        // Pack and transpose: the kernels compute x * W, torch-style gradients are laid out for W * x
+        if (pack_transpose_gradient) net_gradients_.PackAndTranspose(net_gradients_);
+
+        torch::Tensor input_grad;
+        if (get_dl_dinput) input_grad = fromDevice<T>(dL_dinput.GetPointer(), {(int64_t)dL_dinput.nelements(), 1});
+        return {input_grad, fromDevice<T>(net_gradients_.GetViews().GetMatrixPointer(0), {(int64_t)net_gradients_.nelements(), 1})};
+    }
+
+    torch::Tensor initialize_params() override { return get_params(); }
+    torch::Tensor get_params() override { return convertDeviceMatricesToTorchTensor(network_.get_weights_matrices()); }
+    torch::Tensor initialize_params(const torch::Tensor &tensor) override {
+        set_params(tensor, false);
+        return initialize_params();
+    }
+
+    size_t n_params() override { return network_.get_weights_matrices().nelements(); }
+    size_t n_output_dims() override { return network_.get_output_width(); }
+
+    /// The parameters stay on the device: a GPU tensor of any floating dtype is converted and (if unpacked)
+    /// packed there. A CPU tensor takes the reference's route through a host vector.
+    void set_params(const torch::Tensor &params, bool weights_are_packed) override {
+        if ((size_t)params.numel() != n_params())
+            throw std::runtime_error("m_weights_matrices nelements: " + std::to_string(n_params()) +
+                                     " does not match unpacked_weights size: " + std::to_string(params.numel()) +
+                                     ". Consider padding input and output to have the same amount as network_width");
+        if (!params.device().is_cuda()) {
+            network_.set_weights_matrices(convertTensorToVector<T>(params), weights_are_packed);
+            return;
+        }
+        const torch::Tensor p = params.contiguous();
+        switch (p.scalar_type()) {
+        case torch::kFloat32: network_.set_weights_matrices_from_device(p.data_ptr<float>(), weights_are_packed); break;
+        case c10::ScalarType::Half:
+            network_.set_weights_matrices_from_device(reinterpret_cast<const fp16 *>(p.data_ptr()), weights_are_packed);
+            break;
+        case c10::ScalarType::BFloat16:
+            network_.set_weights_matrices_from_device(reinterpret_cast<const bf16 *>(p.data_ptr()), weights_are_packed);
+            break;
+        default: throw std::invalid_argument("params must be float32, float16 or bfloat16");
+        }
+    }
+
+    std::vector<T> get_network_params() { return network_.get_weights_matrices().copy_to_host(); }
+    std::vector<T> get_network_grads() { return net_gradients_.copy_to_host(); }
+
+  protected:
+    void AllocateWorkspace(const size_t batch_size) override {
+        if (batch_size > max_batch_size_) {
+            this->get_queue().wait();
+            this->FreeWorkspace();
+            const size_t in_w = network_.get_input_width(), out_w = network_.get_output_width(), w = network_.get_network_width(),
+                         l = network_.get_n_hidden_layers();
+            interm_forw_ptr_ = tnn::detail::device_alloc<T>(batch_size * (in_w + out_w + w * l));
+            interm_backw_ptr_ = tnn::detail::device_alloc<T>(batch_size * (out_w + w * l));
+            dL_dinput_ptr_ = tnn::detail::device_alloc<T>(batch_size * in_w);
+            max_batch_size_ = batch_size;
+        }
+    }
+
+    void FreeWorkspace() override {
+        tnn::detail::device_free(interm_forw_ptr_);
+        interm_forw_ptr_ = nullptr;
+        tnn::detail::device_free(interm_backw_ptr_);
+        interm_backw_ptr_ = nullptr;
+        tnn::detail::device_free(dL_dinput_ptr_);
+        dL_dinput_ptr_ = nullptr;
+        max_batch_size_ = 0;
+        forward_batch_size_ = 0;
+    }
+
+  private:
+    size_t CheckedBatch(const torch::Tensor &input_tensor, const uint32_t width) const {
+        CHECK_INPUT(input_tensor);
+        TORCH_CHECK(input_tensor.dim() == 2, "input_tensor must have two dimensions");
+        TORCH_CHECK(input_tensor.scalar_type() == torch_type<T>::dtype, "input_tensor has the wrong dtype");
+        if (input_tensor.sizes()[1] != width)
+            throw std::invalid_argument("Input array too small. Input n: " + std::to_string(input_tensor.sizes()[1]) + " != input width " +
+                                        std::to_string(width));
+        if (input_tensor.sizes()[0] % 8 != 0) throw std::invalid_argument("Batch size is not divisible by 8.");
+        return input_tensor.sizes()[0];
+    }
+
+    DeviceMatricesView<T> ForwardViews(const size_t batch_size) const {
+        return DeviceMatricesView<T>(network_.get_n_hidden_layers() + 2, batch_size, network_.get_input_width(), batch_size,
+                                     network_.get_network_width(), batch_size, network_.get_output_width(), interm_forw_ptr_);
+    }
+
+    SwiftNetMLP<T, WIDTH> network_;
+    DeviceMatrices<T> net_gradients_; // independent of the batch size
+    size_t max_batch_size_;           // the workspaces fit every batch size seen so far
+    size_t forward_batch_size_ = 0;   // batch size of the activations held in interm_forw_ptr_
+    T *interm_forw_ptr_;
+    T *interm_backw_ptr_;
+    T *dL_dinput_ptr_;
+};
+
+} // namespace tnn

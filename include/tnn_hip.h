@@ -188,6 +188,24 @@ int tnn_mlp_adam_update(const tnn_mlp_desc *desc, float *d_master_packed, float 
                         float grad_scale, int step, float lr, float beta1, float beta2, float eps, void *d_packed_T,
                         void *d_prepared_fwd, void *d_prepared_bwd, tnn_stream_t stream);
 
+/* One whole optimisation step in two launches: tnn_mlp_train_step_l2 whose gradient reduction applies Adam
+ * (tnn_mlp_adam_update's arithmetic, gradients multiplied by 1 / loss_scale) to the reduced sums directly, i.e. the
+ * reference's loss.backward() + optimizer.step() + the weight re-staging of the next forward
+ * (dpcpp_bindings/tiny_dpcpp_nn/modules.py:96-136,184-207 around torch.optim.Adam) without the gradients ever
+ * reaching HBM as a tensor.
+ *   d_prepared_fwd / d_prepared_bwd: read by this step, rewritten with the updated weights for the next one.
+ *   d_master_packed, d_m, d_v: fp32, packed parameter layout, updated in place. step counts from 1.
+ *   d_y, d_loss_sum, d_packed_T, d_dLdx: optional outputs as in the two functions above.
+ *   main_kernel_done_event: NULL, or a hipEvent_t that is recorded on the stream after the step's main kernel
+ *   (forward + loss + backward + partial weight gradients) and before the reduction, so that a caller can time the
+ *   main kernel without a profiler.
+ * Workspace: tnn_mlp_train_step_workspace_bytes. */
+int tnn_mlp_train_step_l2_adam(const tnn_mlp_desc *desc, void *d_prepared_fwd, void *d_prepared_bwd, const void *d_x,
+                               const float *d_targets, float loss_scale, void *d_y, float *d_loss_sum, float *d_master_packed,
+                               float *d_m, float *d_v, int step, float lr, float beta1, float beta2, float eps, void *d_packed_T,
+                               void *d_dLdx, size_t M, void *d_workspace, size_t workspace_bytes, void *main_kernel_done_event,
+                               tnn_stream_t stream);
+
 /* ------------------------------------------------------------------------------------------
  * Multi-resolution hash grid (include/encodings/grid.h, include/common/common_device.h:700-775).
  * ------------------------------------------------------------------------------------------ */

@@ -85,3 +85,56 @@ def test_fused_adam_update_equals_the_three_separate_calls(tnn, dtype, tdt, W, n
                                            ptr(pT2), ptr(f2), ptr(b2), tnn.stream()))
     for a, b in ((p1, p2), (m1, m2), (v1, v2), (pT1, pT2), (f1, f2), (b1, b2)):
         assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("dtype,tdt", [(BF16, torch.bfloat16), (FP16, torch.float16)])
+@pytest.mark.parametrize("W,n_hidden,M", [(64, 4, 8192), (16, 2, 1000 * 8), (32, 5, 4096), (128, 2, 2048), (64, 6, 2048)])
+def test_train_step_with_adam_equals_step_then_update(tnn, dtype, tdt, W, n_hidden, M):
+    """tnn_mlp_train_step_l2_adam == tnn_mlp_train_step_l2 (fp32 gradients) + tnn_mlp_adam_update, bit for bit: the same
+    reduction order produces the same gradient sums, the same per-weight arithmetic follows. Covers shapes with the fused
+    kernel and shapes without one (width 128, or too deep), and two steps in a row (the second reads the re-staged weights)."""
+    import ctypes
+    from gpu_harness import ptr
+    from tiny_dpcpp_nn import _lib
+    n_mats = n_hidden + 1
+    n = n_mats * W * W
+    gen = torch.Generator(device=tnn.dev).manual_seed(W * 7 + n_hidden)
+    desc = tnn.mlp_desc(dtype, W, n_hidden, "relu", "none")
+    d = ctypes.byref(desc)
+    master = (torch.rand(n, device=tnn.dev, generator=gen) * 2 - 1) * (6.0 / (2 * W)) ** 0.5
+    x = (torch.rand((M, W), device=tnn.dev, generator=gen) * 2 - 1).to(tdt)
+    targets = torch.rand((M, W), device=tnn.dev, generator=gen)
+    loss_scale = 128.0 if dtype == FP16 else 1.0
+    ws_bytes = tnn.lib.tnn_mlp_train_step_workspace_bytes(d, M)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=tnn.dev)
+    hyper = (1e-2, 0.9, 0.99, 1e-15)
+
+    def fresh():
+        f, b = tnn.prepare_packed(desc, master, src_is_fp32=True)
+        return dict(p=master.clone(), m=torch.zeros(n, device=tnn.dev), v=torch.zeros(n, device=tnn.dev), f=f, b=b,
+                    pT=torch.empty(n, dtype=tdt, device=tnn.dev), y=torch.empty_like(x), dx=torch.empty_like(x),
+                    loss=torch.zeros(1, device=tnn.dev))
+
+    a, b = fresh(), fresh()
+    dW = torch.empty((n_mats, W, W), device=tnn.dev)
+    for step in (1, 2):
+        _lib.check(tnn.lib.tnn_mlp_train_step_l2(d, ptr(a["f"]), ptr(a["b"]), ptr(x), ptr(targets), loss_scale, ptr(a["y"]), ptr(a["loss"]),
+                                                 ptr(dW), 1, ptr(a["dx"]), M, ptr(ws), ws_bytes, tnn.stream()))
+        _lib.check(tnn.lib.tnn_mlp_adam_update(d, ptr(a["p"]), ptr(a["m"]), ptr(a["v"]), ptr(dW), 1.0 / loss_scale, step, *hyper,
+                                               ptr(a["pT"]), ptr(a["f"]), ptr(a["b"]), tnn.stream()))
+        _lib.check(tnn.lib.tnn_mlp_train_step_l2_adam(d, ptr(b["f"]), ptr(b["b"]), ptr(x), ptr(targets), loss_scale, ptr(b["y"]),
+                                                      ptr(b["loss"]), ptr(b["p"]), ptr(b["m"]), ptr(b["v"]), step, *hyper, ptr(b["pT"]),
+                                                      ptr(b["dx"]), M, ptr(ws), ws_bytes, None, tnn.stream()))
+        torch.cuda.synchronize()
+        for key in ("y", "dx", "p", "m", "v", "pT", "f", "b"):
+            assert torch.equal(a[key], b[key]), f"step {step}: {key} differs"
+        # shapes without the fused kernel add the loss up with float atomics, in an order that changes from run to run
+        assert torch.allclose(a["loss"], b["loss"], rtol=1e-5, atol=0), f"step {step}: loss differs"
+    assert not torch.equal(a["p"], master)   # the weights did move
+    # argument checks
+    assert tnn.lib.tnn_mlp_train_step_l2_adam(d, ptr(b["f"]), ptr(b["b"]), ptr(x), ptr(targets), loss_scale, None, None, ptr(b["p"]),
+                                              ptr(b["m"]), ptr(b["v"]), 0, *hyper, None, None, M, ptr(ws), ws_bytes, None,
+                                              tnn.stream()) == _lib.TNN_ERR_INVALID_ARGUMENT
+    assert tnn.lib.tnn_mlp_train_step_l2_adam(d, ptr(b["f"]), ptr(b["b"]), ptr(x), ptr(targets), loss_scale, None, None, ptr(b["p"]),
+                                              ptr(b["m"]), ptr(b["v"]), 1, *hyper, None, None, M, ptr(ws), 16, None,
+                                              tnn.stream()) == _lib.TNN_ERR_WORKSPACE

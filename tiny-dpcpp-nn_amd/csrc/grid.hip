@@ -109,14 +109,6 @@ __device__ __forceinline__ void cell_of(const float (&x)[D], float scale, uint32
     }
 }
 
-template <typename P> struct TableVec;
-template <> struct TableVec<float> {
-    static __device__ __forceinline__ float ld(const float *p) { return *p; }
-};
-template <> struct TableVec<fp16_t> {
-    static __device__ __forceinline__ float ld(const fp16_t *p) { return (float)*p; }
-};
-
 template <typename P, int F> __device__ __forceinline__ void load_entry(const P *__restrict__ p, float (&v)[F]) {
     // F consecutive features of one entry, fetched as a single vector load
     typedef P vecF __attribute__((ext_vector_type(F)));

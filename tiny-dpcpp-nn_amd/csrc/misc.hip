@@ -1,5 +1,6 @@
 // Error reporting, weight-layout permutations, L2 loss and the Adam step.
 #include "tnn_internal.h"
+#include "adam_update.h"
 
 #include <cstring>
 
@@ -121,31 +122,9 @@ template <typename D, typename S> __global__ void cast_kernel(D *__restrict__ d,
 // One thread per weight: reads the raw gradient element dW[l][n][k], updates the fp32 master copy (packed
 // layout) with Adam, and writes the rounded weight to the packed T copy and to both operand-order copies.
 template <typename T>
-__global__ void __launch_bounds__(256)
-    mlp_adam_update_kernel(float *__restrict__ master, float *__restrict__ m, float *__restrict__ v, const float *__restrict__ dW_raw,
-                           float grad_scale, int W, int n_mats, float step_size, float bc2_sqrt, float beta1, float beta2, float eps,
-                           T *__restrict__ packed_T, T *__restrict__ prep_fwd, T *__restrict__ prep_bwd) {
+__global__ void __launch_bounds__(256) mlp_adam_update_kernel(const AdamArgs a, const float *__restrict__ dW_raw, int total) {
     const int idx = blockIdx.x * blockDim.x + threadIdx.x;
-    const int per = W * W;
-    if (idx >= per * n_mats) return;
-    const int l = idx / per, e = idx % per;
-    const int n = e / W, k = e % W; // raw gradients are [n = out][k = in]
-    const int pidx = l * per + packed_coord(k, n, W);
-    const float g = dW_raw[idx] * grad_scale;
-    const float mi = m[pidx] + (1.0f - beta1) * (g - m[pidx]);
-    const float vi = beta2 * v[pidx] + (1.0f - beta2) * g * g;
-    m[pidx] = mi;
-    v[pidx] = vi;
-    const float denom = sqrtf(vi) / bc2_sqrt + eps;
-    const float p = master[pidx] - step_size * (mi / denom);
-    master[pidx] = p;
-    const T pt = (T)p;
-    if (packed_T) packed_T[pidx] = pt;
-    const int NI = (W + 31) / 32, NK = W / 16;
-    if (prep_fwd) // product index n, contraction index k
-        prep_fwd[(((size_t)l * NI + n / 32) * NK + k / 16) * 512 + (32 * ((k % 16) / 8) + swap23(n % 32)) * 8 + (k % 8)] = pt;
-    if (prep_bwd) // product index k, contraction index n
-        prep_bwd[(((size_t)l * NI + k / 32) * NK + n / 16) * 512 + (32 * ((n % 16) / 8) + swap23(k % 32)) * 8 + (n % 8)] = pt;
+    if (idx < total) adam_update_element<T>(a, idx, dW_raw[idx]);
 }
 
 } // namespace tnn
@@ -275,21 +254,15 @@ TNN_API int tnn_mlp_adam_update(const tnn_mlp_desc *desc, float *d_master_packed
     if (rc) return rc;
     if (!d_master_packed || !d_m || !d_v || !d_dW_raw) return fail(TNN_ERR_INVALID_ARGUMENT, "NULL pointer argument");
     if (step < 1) return fail(TNN_ERR_INVALID_ARGUMENT, "step counts from 1");
-    const double bc1 = 1.0 - pow((double)beta1, step);
-    const double bc2 = 1.0 - pow((double)beta2, step);
-    const float step_size = (float)(lr / bc1);
-    const float bc2_sqrt = (float)sqrt(bc2);
     const int W = desc->width, n_mats = desc->n_hidden_layers + 1;
     const int total = W * W * n_mats;
+    const AdamArgs a = make_adam_args(d_master_packed, d_m, d_v, grad_scale, step, lr, beta1, beta2, eps, d_packed_T, d_prepared_fwd,
+                                      d_prepared_bwd, W);
     hipStream_t s = as_stream(stream);
     if (desc->dtype == TNN_BF16)
-        TNN_LAUNCH((mlp_adam_update_kernel<bf16_t>), dim3((total + 255) / 256), dim3(256), 0, s, d_master_packed, d_m, d_v, d_dW_raw,
-                           grad_scale, W, n_mats, step_size, bc2_sqrt, beta1, beta2, eps, (bf16_t *)d_packed_T, (bf16_t *)d_prepared_fwd,
-                           (bf16_t *)d_prepared_bwd);
+        TNN_LAUNCH((mlp_adam_update_kernel<bf16_t>), dim3((total + 255) / 256), dim3(256), 0, s, a, d_dW_raw, total);
     else
-        TNN_LAUNCH((mlp_adam_update_kernel<fp16_t>), dim3((total + 255) / 256), dim3(256), 0, s, d_master_packed, d_m, d_v, d_dW_raw,
-                           grad_scale, W, n_mats, step_size, bc2_sqrt, beta1, beta2, eps, (fp16_t *)d_packed_T, (fp16_t *)d_prepared_fwd,
-                           (fp16_t *)d_prepared_bwd);
+        TNN_LAUNCH((mlp_adam_update_kernel<fp16_t>), dim3((total + 255) / 256), dim3(256), 0, s, a, d_dW_raw, total);
     return check_launch("mlp_adam_update_kernel");
 }
 

@@ -60,13 +60,13 @@ __global__ void prepare_weights_kernel(const SRC *__restrict__ packed, T *__rest
 // ACT (hidden activation) is a compile-time constant so that the layer loop stays one basic block:
 // the fragments of the next matrix are requested from LDS before the current accumulators are
 // converted, and arrive while the conversion runs.
-template <typename T, int W, int ACT, bool STORE_INTERM, bool W_IN_LDS, int THREADS, bool PREFETCH>
+template <typename T, int W, int ACT, bool STORE_INTERM, bool W_IN_LDS, int THREADS>
 __global__ void __launch_bounds__(THREADS, (THREADS == 512 && W <= 64) ? 4 : 1)
     mlp_forward_kernel(const typename Storage<T>::vec8 *__restrict__ wprep, const T *__restrict__ x, T *__restrict__ out,
                        int n_mats, int out_act, long long M) {
     typedef Tile<T, W> TL;
     typedef typename Storage<T>::vec8 vec8;
-    constexpr int NK = TL::NK, NI = TL::NI, NF = TL::NF;
+    constexpr int NK = TL::NK, NI = TL::NI;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     vec8 *lds_w = reinterpret_cast<vec8 *>(smem_raw);
 
@@ -88,42 +88,17 @@ __global__ void __launch_bounds__(THREADS, (THREADS == 512 && W <= 64) ? 4 : 1)
         // prefetch the next tile of this wave while the current one is being computed
         const long long next_tile = tile + stride;
         vec8 nxt[NK];
-#ifdef EXP_NO_LOAD
-        if (next_tile < n_tiles) { for (int kb = 0; kb < NK; ++kb) nxt[kb] = cur[kb]; }
-#else
         if (next_tile < n_tiles) TL::load(nxt, x, next_tile * 32 + j, h, next_tile * 32 + j < M);
-#endif
 
         if (STORE_INTERM) TL::store(cur, out, row, h, valid);
         f32x16 acc[NI];
-#ifdef EXP_NO_COMPUTE
-        if (n_mats < 0)
-#endif
-        if constexpr (NF <= 8 && PREFETCH) {
-            // all fragments of a matrix fit in registers: request matrix l+1 before converting layer l
-            vec8 frag[NF];
-            TL::load_frags(frag, wsrc, 0, lane);
-            for (int l = 0; l < n_mats - 1; ++l) {
-                TL::mma(acc, cur, frag);
-                TL::load_frags(frag, wsrc, l + 1, lane);
-                TL::template repack<ACT>(cur, acc);
-                if (STORE_INTERM) TL::store(cur, out + (size_t)(l + 1) * M * W, row, h, valid);
-            }
-            TL::mma(acc, cur, frag);
-        } else {
-            for (int l = 0; l < n_mats - 1; ++l) {
-                TL::template matmul<W_IN_LDS>(acc, cur, lds_w, wprep, l, lane);
-                TL::template repack<ACT>(cur, acc);
-                if (STORE_INTERM) TL::store(cur, out + (size_t)(l + 1) * M * W, row, h, valid);
-            }
-            TL::template matmul<W_IN_LDS>(acc, cur, lds_w, wprep, n_mats - 1, lane);
+        for (int l = 0; l < n_mats - 1; ++l) {
+            TL::template matmul<W_IN_LDS>(acc, cur, lds_w, wprep, l, lane);
+            TL::template repack<ACT>(cur, acc);
+            if (STORE_INTERM) TL::store(cur, out + (size_t)(l + 1) * M * W, row, h, valid);
         }
-#ifndef EXP_NO_COMPUTE
+        TL::template matmul<W_IN_LDS>(acc, cur, lds_w, wprep, n_mats - 1, lane);
         TL::repack_rt(cur, acc, out_act);
-#endif
-#ifdef EXP_NO_STORE
-        if (cur[0][0] == (T)123.25f)
-#endif
         TL::store(cur, STORE_INTERM ? out + (size_t)n_mats * M * W : out, row, h, valid);
 
         if (next_tile < n_tiles) {
@@ -362,7 +337,7 @@ static long long stream_grid(const void *kernel, size_t lds_bytes, size_t M, int
     return blocks < 1 ? 1 : blocks;
 }
 
-template <typename T, int W, int ACT, bool STORE_INTERM, int THREADS, bool PREFETCH>
+template <typename T, int W, int ACT, bool STORE_INTERM, int THREADS>
 static int launch_forward_v(const tnn_mlp_desc *d, const void *wprep, const void *x, void *out, size_t M, hipStream_t s, int per_cu) {
     typedef typename Storage<T>::vec8 vec8;
     const int n_mats = d->n_hidden_layers + 1;
@@ -377,7 +352,7 @@ static int launch_forward_v(const tnn_mlp_desc *d, const void *wprep, const void
     if (blocks > (long long)di.n_cu * per_cu) blocks = (long long)di.n_cu * per_cu;
     if (blocks < 1) blocks = 1;
     if (in_lds) {
-        auto k = mlp_forward_kernel<T, W, ACT, STORE_INTERM, true, THREADS, PREFETCH>;
+        auto k = mlp_forward_kernel<T, W, ACT, STORE_INTERM, true, THREADS>;
         if (wbytes > 48 * 1024 &&
             hipFuncSetAttribute(reinterpret_cast<const void *>(k), hipFuncAttributeMaxDynamicSharedMemorySize,
                                 (int)wbytes) != hipSuccess)
@@ -385,24 +360,19 @@ static int launch_forward_v(const tnn_mlp_desc *d, const void *wprep, const void
         TNN_LAUNCH(k, dim3((unsigned)blocks), dim3(THREADS), wbytes, s, (const vec8 *)wprep, (const T *)x,
                            (T *)out, n_mats, d->output_activation, (long long)M);
     } else {
-        auto k = mlp_forward_kernel<T, W, ACT, STORE_INTERM, false, THREADS, PREFETCH>;
+        auto k = mlp_forward_kernel<T, W, ACT, STORE_INTERM, false, THREADS>;
         TNN_LAUNCH(k, dim3((unsigned)blocks), dim3(THREADS), 0, s, (const vec8 *)wprep, (const T *)x, (T *)out,
                            n_mats, d->output_activation, (long long)M);
     }
     return check_launch("mlp_forward_kernel");
 }
 
+// 512 threads (8 waves, one 32-row tile each at a time) and two workgroups per CU: at most 128 VGPRs per lane,
+// measured faster than 256-thread workgroups at higher counts and than variants that hold the next matrix's
+// fragments in registers.
 template <typename T, int W, int ACT, bool STORE_INTERM>
 static int launch_forward_act(const tnn_mlp_desc *d, const void *wprep, const void *x, void *out, size_t M, hipStream_t s) {
-    static const char *ev = getenv("TNN_FWD_VARIANT");
-    const int v = ev ? atoi(ev) : 0;
-    switch (v) {
-    case 1: return launch_forward_v<T, W, ACT, STORE_INTERM, 512, true>(d, wprep, x, out, M, s, 2);
-    case 2: return launch_forward_v<T, W, ACT, STORE_INTERM, 256, true>(d, wprep, x, out, M, s, 3);
-    case 3: return launch_forward_v<T, W, ACT, STORE_INTERM, 256, false>(d, wprep, x, out, M, s, 4);
-    case 4: return launch_forward_v<T, W, ACT, STORE_INTERM, 256, false>(d, wprep, x, out, M, s, 3);
-    default: return launch_forward_v<T, W, ACT, STORE_INTERM, 512, false>(d, wprep, x, out, M, s, 2);
-    }
+    return launch_forward_v<T, W, ACT, STORE_INTERM, 512>(d, wprep, x, out, M, s, 2);
 }
 
 template <typename T, int W, bool STORE_INTERM>

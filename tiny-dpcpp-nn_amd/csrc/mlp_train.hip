@@ -40,7 +40,8 @@ FusedPlan fused_plan(const tnn_mlp_desc *d, size_t M) {
 
 // Used by tnn_mlp_train_step_l2: returns TNN_ERR_UNSUPPORTED when the shape has no fused kernel.
 int fused_train_step(const tnn_mlp_desc *d, const void *wf, const void *wb, const void *x, const float *targets, float loss_scale,
-                     void *y, float *loss_sum, void *dW, int dW_is_fp32, void *dx, size_t M, void *ws, size_t ws_bytes, hipStream_t s) {
+                     void *y, float *loss_sum, void *dW, int dW_is_fp32, void *dx, size_t M, void *ws, size_t ws_bytes, const TrainTail &tail,
+                     hipStream_t s) {
     const FusedPlan p = fused_plan(d, M);
     if (!p.supported) return TNN_ERR_UNSUPPORTED;
     const size_t need = p.partial_bytes + p.loss_bytes + 512;
@@ -49,8 +50,8 @@ int fused_train_step(const tnn_mlp_desc *d, const void *wf, const void *wb, cons
     float *loss_partials = reinterpret_cast<float *>(base);
     float *partials = reinterpret_cast<float *>(base + p.loss_bytes);
     if (d->dtype == TNN_BF16)
-        return fused_train_launch_bf16(d, p, wf, wb, x, targets, loss_scale, y, loss_sum, dW, dW_is_fp32, dx, M, partials, loss_partials, s);
-    return fused_train_launch_fp16(d, p, wf, wb, x, targets, loss_scale, y, loss_sum, dW, dW_is_fp32, dx, M, partials, loss_partials, s);
+        return fused_train_launch_bf16(d, p, wf, wb, x, targets, loss_scale, y, loss_sum, dW, dW_is_fp32, dx, M, partials, loss_partials, tail, s);
+    return fused_train_launch_fp16(d, p, wf, wb, x, targets, loss_scale, y, loss_sum, dW, dW_is_fp32, dx, M, partials, loss_partials, tail, s);
 }
 
 // 0 when the shape has no fused kernel

@@ -4,7 +4,7 @@
 namespace tnn {
 int fused_train_launch_bf16(const tnn_mlp_desc *d, const FusedPlan &p, const void *wf, const void *wb, const void *x,
                             const float *targets, float loss_scale, void *y, float *loss_sum, void *dW, int dW_is_fp32, void *dx,
-                            size_t M, float *partials, float *loss_partials, hipStream_t s) {
-    return launch_fused_w<bf16_t>(d, p, wf, wb, x, targets, loss_scale, y, loss_sum, dW, dW_is_fp32, dx, M, partials, loss_partials, s);
+                            size_t M, float *partials, float *loss_partials, const TrainTail &tail, hipStream_t s) {
+    return launch_fused_w<bf16_t>(d, p, wf, wb, x, targets, loss_scale, y, loss_sum, dW, dW_is_fp32, dx, M, partials, loss_partials, tail, s);
 }
 } // namespace tnn

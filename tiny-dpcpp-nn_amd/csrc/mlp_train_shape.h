@@ -1,6 +1,7 @@
 // Shape constants and the launch plan of the fused training-step kernel.
 #pragma once
 
+#include "adam_update.h"
 #include "mlp_tile.h"
 
 namespace tnn {
@@ -34,9 +35,9 @@ FusedPlan fused_plan(const tnn_mlp_desc *d, size_t M);
 // per storage type (mlp_train_bf16.hip / mlp_train_fp16.hip)
 int fused_train_launch_bf16(const tnn_mlp_desc *d, const FusedPlan &p, const void *wf, const void *wb, const void *x,
                             const float *targets, float loss_scale, void *y, float *loss_sum, void *dW, int dW_is_fp32, void *dx,
-                            size_t M, float *partials, float *loss_partials, hipStream_t s);
+                            size_t M, float *partials, float *loss_partials, const TrainTail &tail, hipStream_t s);
 int fused_train_launch_fp16(const tnn_mlp_desc *d, const FusedPlan &p, const void *wf, const void *wb, const void *x,
                             const float *targets, float loss_scale, void *y, float *loss_sum, void *dW, int dW_is_fp32, void *dx,
-                            size_t M, float *partials, float *loss_partials, hipStream_t s);
+                            size_t M, float *partials, float *loss_partials, const TrainTail &tail, hipStream_t s);
 
 } // namespace tnn

@@ -1,5 +1,6 @@
 // One training step of the fused MLP against an L2 loss: forward, loss + gradient, backward with
 // weight gradients (include/trainer.h:23-46 with include/losses/l2.h:19-40 in between).
+#include "adam_update.h"
 #include "tnn_internal.h"
 
 namespace tnn {
@@ -28,10 +29,12 @@ __global__ void __launch_bounds__(256)
 __global__ void zero_scalar_kernel(float *p) { *p = 0.0f; }
 
 static size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
+static size_t unfused_dw_bytes(const tnn_mlp_desc *d) { return (size_t)(d->n_hidden_layers + 1) * d->width * d->width * sizeof(float); }
 
 // mlp_train.hip
 int fused_train_step(const tnn_mlp_desc *d, const void *wf, const void *wb, const void *x, const float *targets, float loss_scale,
-                     void *y, float *loss_sum, void *dW, int dW_is_fp32, void *dx, size_t M, void *ws, size_t ws_bytes, hipStream_t s);
+                     void *y, float *loss_sum, void *dW, int dW_is_fp32, void *dx, size_t M, void *ws, size_t ws_bytes, const TrainTail &tail,
+                     hipStream_t s);
 size_t fused_train_workspace_bytes(const tnn_mlp_desc *d, size_t M);
 
 } // namespace tnn
@@ -43,7 +46,9 @@ TNN_API size_t tnn_mlp_train_step_workspace_bytes(const tnn_mlp_desc *desc, size
     const size_t fused = fused_train_workspace_bytes(desc, M);
     if (fused) return fused;
     const size_t mat = M * desc->width * 2;
-    return align256((size_t)(desc->n_hidden_layers + 2) * mat) + align256(mat) + tnn_mlp_backward_workspace_bytes(desc, M) + 512;
+    // activations, dL/dy, the backward pass's own workspace, and fp32 weight gradients for tnn_mlp_train_step_l2_adam
+    return align256((size_t)(desc->n_hidden_layers + 2) * mat) + align256(mat) + align256(tnn_mlp_backward_workspace_bytes(desc, M)) +
+           align256(unfused_dw_bytes(desc)) + 512;
 }
 
 TNN_API int tnn_mlp_train_step_l2(const tnn_mlp_desc *desc, const void *d_prepared_fwd, const void *d_prepared_bwd,
@@ -61,7 +66,7 @@ TNN_API int tnn_mlp_train_step_l2(const tnn_mlp_desc *desc, const void *d_prepar
     if (M == 0 || (M % 8) != 0) return fail(TNN_ERR_INVALID_ARGUMENT, "batch size %zu is not a positive multiple of 8", M);
     // shapes with a fused kernel never touch device memory with activations or deltas
     rc = fused_train_step(desc, d_prepared_fwd, d_prepared_bwd, d_x, d_targets, loss_scale, d_y, d_loss_sum, d_dW, dW_is_fp32, d_dLdx, M,
-                          d_workspace, workspace_bytes, s);
+                          d_workspace, workspace_bytes, TrainTail{}, s);
     if (rc != TNN_ERR_UNSUPPORTED) return rc;
     // wider / deeper networks: forward, loss and backward as separate kernels over workspace matrices
     const int W = desc->width, n_mats = desc->n_hidden_layers + 1;
@@ -72,7 +77,7 @@ TNN_API int tnn_mlp_train_step_l2(const tnn_mlp_desc *desc, const void *d_prepar
     void *dLdy = reinterpret_cast<void *>(base);
     base += align256(mat);
     void *bwd_ws = reinterpret_cast<void *>(base);
-    const size_t bwd_ws_bytes = workspace_bytes - (base - reinterpret_cast<uintptr_t>(d_workspace));
+    const size_t bwd_ws_bytes = align256(tnn_mlp_backward_workspace_bytes(desc, M));
 
     if ((rc = tnn_mlp_forward(desc, d_prepared_fwd, d_x, interm_fwd, M, stream))) return rc;
     const void *y = static_cast<const char *>(interm_fwd) + (size_t)n_mats * mat;
@@ -90,4 +95,40 @@ TNN_API int tnn_mlp_train_step_l2(const tnn_mlp_desc *desc, const void *d_prepar
                            loss_scale, d_loss_sum, (fp16_t *)dLdy);
     if ((rc = check_launch("l2_loss_sum_kernel"))) return rc;
     return tnn_mlp_backward(desc, d_prepared_bwd, dLdy, interm_fwd, nullptr, d_dW, dW_is_fp32, d_dLdx, M, bwd_ws, bwd_ws_bytes, stream);
+}
+
+TNN_API int tnn_mlp_train_step_l2_adam(const tnn_mlp_desc *desc, void *d_prepared_fwd, void *d_prepared_bwd, const void *d_x,
+                                       const float *d_targets, float loss_scale, void *d_y, float *d_loss_sum, float *d_master_packed,
+                                       float *d_m, float *d_v, int step, float lr, float beta1, float beta2, float eps,
+                                       void *d_packed_T, void *d_dLdx, size_t M, void *d_workspace, size_t workspace_bytes,
+                                       void *main_kernel_done_event, tnn_stream_t stream) {
+    int rc = check_mlp_desc(desc);
+    if (rc) return rc;
+    if (!d_prepared_fwd || !d_prepared_bwd || !d_x || !d_targets || !d_master_packed || !d_m || !d_v)
+        return fail(TNN_ERR_INVALID_ARGUMENT, "NULL pointer argument");
+    if (loss_scale == 0.0f) return fail(TNN_ERR_INVALID_ARGUMENT, "loss_scale must not be 0");
+    if (step < 1) return fail(TNN_ERR_INVALID_ARGUMENT, "step counts from 1");
+    const size_t need = tnn_mlp_train_step_workspace_bytes(desc, M);
+    if (!d_workspace || workspace_bytes < need)
+        return fail(TNN_ERR_WORKSPACE, "workspace of %zu bytes given, %zu needed", workspace_bytes, need);
+    if (M == 0 || (M % 8) != 0) return fail(TNN_ERR_INVALID_ARGUMENT, "batch size %zu is not a positive multiple of 8", M);
+    hipStream_t s = as_stream(stream);
+    TrainTail tail;
+    tail.use_adam = true;
+    tail.adam = make_adam_args(d_master_packed, d_m, d_v, 1.0f / loss_scale, step, lr, beta1, beta2, eps, d_packed_T, d_prepared_fwd,
+                               d_prepared_bwd, desc->width);
+    tail.main_done = static_cast<hipEvent_t>(main_kernel_done_event);
+    rc = fused_train_step(desc, d_prepared_fwd, d_prepared_bwd, d_x, d_targets, loss_scale, d_y, d_loss_sum, nullptr, 1, d_dLdx, M,
+                          d_workspace, workspace_bytes, tail, s);
+    if (rc != TNN_ERR_UNSUPPORTED) return rc;
+    // no fused kernel for this shape: the separate step, then the separate update, over gradients kept in the workspace
+    const uintptr_t end = reinterpret_cast<uintptr_t>(d_workspace) + workspace_bytes;
+    float *dW = reinterpret_cast<float *>((end - unfused_dw_bytes(desc)) & ~(uintptr_t)255);
+    // (the step lays its matrices out from the front of the workspace and stays clear of this tail)
+    if ((rc = tnn_mlp_train_step_l2(desc, d_prepared_fwd, d_prepared_bwd, d_x, d_targets, loss_scale, d_y, d_loss_sum, dW, 1, d_dLdx, M,
+                                    d_workspace, workspace_bytes, stream)))
+        return rc;
+    if (tail.main_done && hipEventRecord(tail.main_done, s) != hipSuccess) return fail(TNN_ERR_HIP, "hipEventRecord failed");
+    return tnn_mlp_adam_update(desc, d_master_packed, d_m, d_v, dW, 1.0f / loss_scale, step, lr, beta1, beta2, eps, d_packed_T,
+                               d_prepared_fwd, d_prepared_bwd, stream);
 }

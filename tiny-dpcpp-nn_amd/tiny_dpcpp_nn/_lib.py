@@ -94,6 +94,11 @@ SIGNATURES = {
         [POINTER(MlpDesc), c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_int, c_float, c_float, c_float, c_float, c_void_p,
          c_void_p, c_void_p, c_void_p],
     ),
+    "tnn_mlp_train_step_l2_adam": (
+        c_int,
+        [POINTER(MlpDesc), c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
+         c_float, c_float, c_float, c_float, c_void_p, c_void_p, c_size_t, c_void_p, c_size_t, c_void_p, c_void_p],
+    ),
     "tnn_grid_desc_init": (
         c_int,
         [POINTER(GridDesc), c_uint32, c_uint32, c_uint32, c_uint32, c_uint32, c_float, c_uint32, c_uint32, c_uint32, c_uint32],

@@ -25,6 +25,16 @@ sys.path.insert(0, os.path.join(ROOT, "tests"))
 PEAK_MFMA_BF16 = 2500.0  # TFLOP/s, dense
 PEAK_HBM = 8000.0  # GB/s
 
+# HBM-side bytes per launch of each workload's dominant kernel at the default batch sizes, from rocprofv3 counter runs over this
+# file (FETCH_SIZE and WRITE_SIZE, one run each, scaled by what the same counter reads for the --copy-calibration kernel:
+# x2.000 and x1.000). The summaries with the commands are profiles/mlp_train_fused_kernel.*.txt, profiles/mlp_forward_kernel.*.txt
+# and profiles/grid_forward_kernel.*.txt. Not measured live: counters need the profiler.
+MEASURED_TRAFFIC_BYTES = {
+    ("train", 18): (57794.4 * 2.0 + 20488.0) * 1024,
+    ("infer", 18): (16573.3 * 2.0 + 32768.0) * 1024,
+    ("grid", 21): (6156642.8 * 2.0 + 262143.8) * 1024,
+}
+
 
 def parse():
     ap = argparse.ArgumentParser()
@@ -34,6 +44,9 @@ def parse():
     ap.add_argument("--workload", default="train", choices=["train", "infer", "grid"])
     ap.add_argument("--batch-log2", type=int, default=None)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also launch a plain copy kernel (tnn_cast fp32 -> fp32, 256 MiB read + 256 MiB written per launch) so that "
+                         "hardware byte counters collected over this run can be scaled by what they read for a known transfer")
     return ap.parse_args()
 
 
@@ -206,7 +219,8 @@ def main():
             "config": {"workload": f"training step: w64, 4 hidden layers (5 matmuls), ReLU/linear, bf16, batch 2^{int(np.log2(M))}, "
                                    "L2 loss, Adam on fp32 masters (BASELINE config 2)", "batch": M},
             "roofline": {"bound": "mfma", "achieved": flops / (kern_ms * 1e-3) / 1e12, "peak": PEAK_MFMA_BF16, "unit": "TFLOP/s",
-                         "frac": flops / (kern_ms * 1e-3) / 1e12 / PEAK_MFMA_BF16, "traffic": None,
+                         "frac": flops / (kern_ms * 1e-3) / 1e12 / PEAK_MFMA_BF16,
+                         "traffic": MEASURED_TRAFFIC_BYTES.get(("train", int(np.log2(M)))),
                          "kernel": "mlp_train_fused_kernel (forward + loss + backward + partial dW)", "kernel_ms": kern_ms,
                          "algorithmic_flops_per_launch": flops},
             "mfma_frac_whole_step": flops / (ms * 1e-3) / 1e12 / PEAK_MFMA_BF16,
@@ -239,7 +253,8 @@ def main():
             "config": {"workload": f"inference: w64, 4 hidden layers (5 matmuls), ReLU/linear, bf16, batch 2^{int(np.log2(M))} (BASELINE config 1 shape)",
                        "batch": M},
             "roofline": {"bound": "hbm", "achieved": bytes_ / (ms * 1e-3) / 1e9, "peak": PEAK_HBM, "unit": "GB/s",
-                         "frac": bytes_ / (ms * 1e-3) / 1e9 / PEAK_HBM, "traffic": None, "kernel": "mlp_forward_kernel (inference)",
+                         "frac": bytes_ / (ms * 1e-3) / 1e9 / PEAK_HBM, "traffic": MEASURED_TRAFFIC_BYTES.get(("infer", int(np.log2(M)))),
+                         "kernel": "mlp_forward_kernel (inference)",
                          "kernel_ms": ms, "algorithmic_bytes_per_launch": bytes_},
             "mfma_frac": flops / (ms * 1e-3) / 1e12 / PEAK_MFMA_BF16,
         }
@@ -274,11 +289,20 @@ def main():
             "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
             "config": {"workload": f"3-D hash-grid encoding forward, 2^{int(np.log2(M))} points (BASELINE config 5 encoding)", "batch": M},
             "roofline": {"bound": "hbm", "achieved": bpp * M / (ms * 1e-3) / 1e9, "peak": PEAK_HBM, "unit": "GB/s",
-                         "frac": bpp * M / (ms * 1e-3) / 1e9 / PEAK_HBM, "traffic": None, "kernel": "grid_forward_kernel",
+                         "frac": bpp * M / (ms * 1e-3) / 1e9 / PEAK_HBM, "traffic": MEASURED_TRAFFIC_BYTES.get(("grid", int(np.log2(M)))),
+                         "kernel": "grid_forward_kernel",
                          "kernel_ms": ms, "algorithmic_bytes_per_launch": bpp * M},
         }
         if oracle is not None:
             out["cpu_baseline"] = cpu_baseline_grid(oracle, cfg)
+
+    if args.copy_calibration:
+        n = 64 << 20
+        src = torch.ones(n, dtype=torch.float32, device=t.dev)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            _lib.check(lib.tnn_cast(FP32, ptr(dst), FP32, ptr(src), n, t.stream()))
+        torch.cuda.synchronize()
 
     print(json.dumps(out))
 

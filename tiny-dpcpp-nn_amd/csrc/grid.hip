@@ -253,31 +253,28 @@ __global__ void __launch_bounds__(kGridThreads)
     }
 }
 
-// One thread per (point, level): levels are the slow grid dimension so that concurrently running
-// workgroups hit the same level's slice of the gradient table (it stays in L2 while it is hot).
-template <int D, int F, typename G>
-__global__ void __launch_bounds__(kGridThreads)
-    grid_backward_kernel(const GridLevels lv, const GridParams gp, const float *__restrict__ xin, const G *__restrict__ dLdy,
-                         float *__restrict__ grad, long long M) {
-    const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i >= M) return;
-    const uint32_t l = blockIdx.y;
-    float x[D];
-#pragma unroll
-    for (int d = 0; d < D; ++d) x[d] = xin[i * D + d];
-    float gy[F];
-#pragma unroll
-    for (int f = 0; f < F; ++f) gy[f] = (float)dLdy[i * gp.padded_width + l * F + f];
+// Which levels the backward pass accumulates in LDS first, and how the 1-D grid is split between the two routes.
+struct BackwardPlan {
+    uint32_t n_small;          // levels whose whole gradient slice fits the LDS budget
+    uint32_t small_blocks;     // workgroups per such level, each takes `chunk` consecutive points
+    uint32_t chunk;
+    uint32_t big_blocks;       // workgroups per other level, one point per thread
+    uint8_t small_level[TNN_GRID_MAX_LEVELS];
+    uint8_t big_level[TNN_GRID_MAX_LEVELS];
+};
 
-    const uint32_t size = lv.size[l], res = lv.resolution[l], flags = lv.flags[l];
-    float *g = grad + (size_t)lv.offset[l] * F;
+constexpr uint32_t kPrivateLdsBytes = 64 * 1024; // per workgroup; two such workgroups fit a CU
+constexpr uint32_t kPrivateChunk = 4096;         // points per workgroup on the LDS route
+
+// Gradient contributions of one point to one level: visits (entry index, weight) of every corner.
+template <int D, typename Fn>
+__device__ __forceinline__ void for_each_corner(const float (&x)[D], float scale, uint32_t size, uint32_t res, uint32_t flags,
+                                                uint32_t hash_type, uint32_t interpolation, Fn &&fn) {
     uint32_t cell[D];
     float frac[D];
-    cell_of<D>(x, lv.scale[l], gp.interpolation, cell, frac);
-    if (gp.interpolation == TNN_INTERP_NEAREST) {
-        const uint32_t idx = level_index<D>(cell, size, res, flags, gp.hash_type);
-#pragma unroll
-        for (int f = 0; f < F; ++f) unsafeAtomicAdd(g + (size_t)idx * F + f, gy[f]);
+    cell_of<D>(x, scale, interpolation, cell, frac);
+    if (interpolation == TNN_INTERP_NEAREST) {
+        fn(level_index<D>(cell, size, res, flags, hash_type), 1.0f);
         return;
     }
 #pragma unroll
@@ -294,10 +291,68 @@ __global__ void __launch_bounds__(kGridThreads)
                 loc[d] = cell[d] + 1;
             }
         }
-        const uint32_t idx = level_index<D>(loc, size, res, flags, gp.hash_type);
-#pragma unroll
-        for (int f = 0; f < F; ++f) unsafeAtomicAdd(g + (size_t)idx * F + f, weight * gy[f]);
+        fn(level_index<D>(loc, size, res, flags, hash_type), weight);
     }
+}
+
+// Scatter-add of dL/dy into the gradient table (include/encodings/grid.h:137-245 of the reference: float atomics,
+// order not defined). Two routes inside one launch:
+//   * small levels (the coarse ones, where every point of the batch lands on a few hundred entries and global
+//     atomics queue up on the same addresses): a workgroup adds the contributions of a chunk of points into a
+//     private copy of the level in LDS and then issues one global atomic per touched entry;
+//   * the other levels: one thread per (point, level), atomics straight to the table; workgroups of one level
+//     are dispatched together, so its slice of the table is the hot one in L2.
+template <int D, int F, typename G>
+__global__ void __launch_bounds__(kGridThreads)
+    grid_backward_kernel(const GridLevels lv, const GridParams gp, const BackwardPlan bp, const float *__restrict__ xin,
+                         const G *__restrict__ dLdy, float *__restrict__ grad, long long M) {
+    extern __shared__ float priv[];
+    const uint32_t n_small_blocks = bp.n_small * bp.small_blocks;
+    if (blockIdx.x < n_small_blocks) {
+        const uint32_t l = bp.small_level[blockIdx.x / bp.small_blocks];
+        const uint32_t size = lv.size[l], res = lv.resolution[l], flags = lv.flags[l];
+        const float scale = lv.scale[l];
+        const uint32_t n = size * F;
+        for (uint32_t e = threadIdx.x; e < n; e += kGridThreads) priv[e] = 0.0f;
+        __syncthreads();
+        const long long first = (long long)(blockIdx.x % bp.small_blocks) * bp.chunk;
+        const long long last = first + bp.chunk < M ? first + bp.chunk : M;
+        for (long long i = first + threadIdx.x; i < last; i += kGridThreads) {
+            float x[D];
+#pragma unroll
+            for (int d = 0; d < D; ++d) x[d] = xin[i * D + d];
+            float gy[F];
+#pragma unroll
+            for (int f = 0; f < F; ++f) gy[f] = (float)dLdy[i * gp.padded_width + l * F + f];
+            for_each_corner<D>(x, scale, size, res, flags, gp.hash_type, gp.interpolation, [&](uint32_t idx, float w) {
+#pragma unroll
+                for (int f = 0; f < F; ++f) atomicAdd(&priv[idx * F + f], w * gy[f]);
+            });
+        }
+        __syncthreads();
+        float *g = grad + (size_t)lv.offset[l] * F;
+        for (uint32_t e = threadIdx.x; e < n; e += kGridThreads) {
+            const float v = priv[e];
+            if (v != 0.0f) unsafeAtomicAdd(g + e, v);
+        }
+        return;
+    }
+    const uint32_t b = blockIdx.x - n_small_blocks;
+    const uint32_t l = bp.big_level[b / bp.big_blocks];
+    const long long i = (long long)(b % bp.big_blocks) * kGridThreads + threadIdx.x;
+    if (i >= M) return;
+    float x[D];
+#pragma unroll
+    for (int d = 0; d < D; ++d) x[d] = xin[i * D + d];
+    float gy[F];
+#pragma unroll
+    for (int f = 0; f < F; ++f) gy[f] = (float)dLdy[i * gp.padded_width + l * F + f];
+    float *g = grad + (size_t)lv.offset[l] * F;
+    for_each_corner<D>(x, lv.scale[l], lv.size[l], lv.resolution[l], lv.flags[l], gp.hash_type, gp.interpolation,
+                       [&](uint32_t idx, float w) {
+#pragma unroll
+                           for (int f = 0; f < F; ++f) unsafeAtomicAdd(g + (size_t)idx * F + f, w * gy[f]);
+                       });
 }
 
 __global__ void fill_zero_kernel(float4 *__restrict__ p, size_t n4, float *__restrict__ tail, size_t n_tail) {
@@ -352,22 +407,41 @@ static int launch_grid_forward_p(const tnn_grid_desc *d, const GridLevels &lv, c
 template <int D, int F>
 static int launch_grid_backward_g(const GridLevels &lv, const GridParams &gp, const float *x, const void *dLdy, int dy_dtype,
                                   float *grad, size_t M, hipStream_t s) {
-    const dim3 grid((unsigned)((M + kGridThreads - 1) / kGridThreads), gp.n_levels);
+    // A level goes the LDS route when its slice fits the budget and a chunk of points makes clearly more atomics
+    // than the flush of the private copy does (chunk * 2^D contributions against `size` entries).
+    BackwardPlan bp{};
+    bp.chunk = kPrivateChunk;
+    bp.small_blocks = (uint32_t)((M + bp.chunk - 1) / bp.chunk);
+    bp.big_blocks = (uint32_t)((M + kGridThreads - 1) / kGridThreads);
+    const size_t per_chunk = (M < bp.chunk ? M : (size_t)bp.chunk) << (gp.interpolation == TNN_INTERP_NEAREST ? 0 : D);
+    uint32_t n_big = 0, lds_bytes = 0;
+    for (uint32_t l = 0; l < gp.n_levels; ++l) {
+        const size_t bytes = (size_t)lv.size[l] * F * sizeof(float);
+        if (bytes <= kPrivateLdsBytes && per_chunk >= 2 * (size_t)lv.size[l]) {
+            bp.small_level[bp.n_small++] = (uint8_t)l;
+            if (bytes > lds_bytes) lds_bytes = (uint32_t)bytes;
+        } else {
+            bp.big_level[n_big++] = (uint8_t)l;
+        }
+    }
+    const unsigned long long blocks = (unsigned long long)bp.n_small * bp.small_blocks + (unsigned long long)n_big * bp.big_blocks;
+    if (blocks > 0x7fffffffull) return fail(TNN_ERR_UNSUPPORTED, "grid backward: batch too large for one launch");
+    const dim3 grid((unsigned)blocks);
+#define TNN_BWD(GT)                                                                                                    \
+    do {                                                                                                               \
+        auto k = grid_backward_kernel<D, F, GT>;                                                                       \
+        if (lds_bytes > 48 * 1024 &&                                                                                   \
+            hipFuncSetAttribute(reinterpret_cast<const void *>(k), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes) != hipSuccess) \
+            return fail(TNN_ERR_HIP, "cannot reserve %u bytes of LDS", lds_bytes);                                     \
+        TNN_LAUNCH(k, grid, dim3(kGridThreads), lds_bytes, s, lv, gp, bp, x, (const GT *)dLdy, grad, (long long)M);    \
+    } while (0)
     switch (dy_dtype) {
-    case TNN_FP32:
-        TNN_LAUNCH((grid_backward_kernel<D, F, float>), grid, dim3(kGridThreads), 0, s, lv, gp, x, (const float *)dLdy, grad,
-                           (long long)M);
-        break;
-    case TNN_BF16:
-        TNN_LAUNCH((grid_backward_kernel<D, F, bf16_t>), grid, dim3(kGridThreads), 0, s, lv, gp, x, (const bf16_t *)dLdy, grad,
-                           (long long)M);
-        break;
-    case TNN_FP16:
-        TNN_LAUNCH((grid_backward_kernel<D, F, fp16_t>), grid, dim3(kGridThreads), 0, s, lv, gp, x, (const fp16_t *)dLdy, grad,
-                           (long long)M);
-        break;
+    case TNN_FP32: TNN_BWD(float); break;
+    case TNN_BF16: TNN_BWD(bf16_t); break;
+    case TNN_FP16: TNN_BWD(fp16_t); break;
     default: return fail(TNN_ERR_UNSUPPORTED, "dy_dtype %d", dy_dtype);
     }
+#undef TNN_BWD
     return check_launch("grid_backward_kernel");
 }
 

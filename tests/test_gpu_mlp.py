@@ -317,3 +317,55 @@ def test_train_step_single_call(tnn, oracle, dtype, W, n_hidden, act, out_act):
     y2, loss2, dW2, dX2 = tnn.train_step_l2(desc, pf, pb, xt, tt, ls, want_y=False, want_dx=False, dw_fp32=False)
     assert y2 is None and dX2 is None
     assert np.array_equal(tnn.host(dW2), oracle.round(dWh, dtype))
+
+
+@pytest.mark.parametrize("W,n_hidden", [(16, 2), (32, 4), (128, 8)])
+def test_baseline_config_3_full_size(tnn, oracle, W, n_hidden):
+    """BASELINE config 3: fp16, batch 2^20, as inference and as a training step. Inference: a seeded sample of 4096 rows
+    against the oracle, and the rows of a sub-batch bit-identical to the same rows inside the full batch. Training step:
+    the loss-scaled weight gradients of the whole batch equal the sum over its two halves (the gradient is additive over
+    rows; fp32 sums in another order), the halves' network outputs are the full batch's rows, and a sampled sub-batch's
+    gradients match the oracle."""
+    import torch
+    dtype, M = FP16, 1 << 20
+    n_mats = n_hidden + 1
+    w = oracle.round(xavier(W, n_mats, 3), dtype)
+    desc = tnn.mlp_desc(dtype, W, n_hidden, "relu", "none")
+    _, pf, pb = tnn.prepare(desc, w)
+    gen = torch.Generator(device=tnn.dev).manual_seed(33)
+    x = (torch.rand((M, W), device=tnn.dev, generator=gen) * 2 - 1).to(torch.float16)
+    y = tnn.inference(desc, pf, x)
+    sel = torch.sort(torch.randperm(M, device=tnn.dev, generator=gen)[:4096]).values
+    ref = oracle.mlp_forward_T(dtype, W, n_mats, "relu", "none", w, x[sel].float().cpu().numpy(), store_interm=False)
+    assert_propagated(y[sel].float().cpu().numpy(), ref, dtype, "config 3 inference, sampled rows")
+    assert torch.equal(tnn.inference(desc, pf, x[4096:3 * 4096].contiguous()), y[4096:3 * 4096])
+
+    targets = torch.rand((M, W), device=tnn.dev, generator=gen)
+    loss_scale = 128.0 * (M / 1024)  # keeps dL/dy = loss_scale * 2 (y - t) / (M W) clear of fp16's denormal range
+    yf, lf, dWf, _ = tnn.train_step_l2(desc, pf, pb, x, targets, loss_scale, want_dx=False)
+    assert torch.equal(yf, y)
+    h = M // 2
+    # a half batch averages over half as many elements: half the loss scale gives the same per-row gradient
+    ya, la, dWa, _ = tnn.train_step_l2(desc, pf, pb, x[:h].contiguous(), targets[:h].contiguous(), loss_scale / 2, want_dx=False)
+    yb, lb, dWb, _ = tnn.train_step_l2(desc, pf, pb, x[h:].contiguous(), targets[h:].contiguous(), loss_scale / 2, want_dx=False)
+    assert torch.equal(ya, y[:h]) and torch.equal(yb, y[h:])
+    full, parts = dWf.double().cpu().numpy(), (dWa.double() + dWb.double()).cpu().numpy()
+    assert np.abs(full - parts).max() <= 1e-4 * np.abs(full).max()
+    assert abs(float(lf) - 0.5 * (float(la) + float(lb))) <= 1e-5 * float(lf)
+    # a sub-batch small enough for the oracle
+    S = 2048
+    xs, ts = x[:S].contiguous(), targets[:S].contiguous()
+    ys_, ls, dWs, dXs = tnn.train_step_l2(desc, pf, pb, xs, ts, 4096.0)
+    interm = oracle.mlp_forward_T(dtype, W, n_mats, "relu", "none", w, xs.float().cpu().numpy())
+    _, grads = oracle.l2_loss(dtype, interm[-1], ts.cpu().numpy(), 4096.0)
+    _, rdW, rdX = oracle.mlp_backward_T(dtype, W, n_mats, "relu", "none", w, interm, grads, round_dw=False)
+    assert_propagated(dWs.cpu().numpy(), rdW, dtype, "dW of the sub-batch", scale=float(np.abs(rdW).max()))
+    # dL/dx has up to nine rounded ReLU layers behind it, forward and backward (the step does not expose its activations,
+    # so the oracle runs on its own), and no sum over the batch to average a flipped mask out: a row in which one
+    # pre-activation rounds to the other side of zero gets the other mask and differs in all of its elements (0.5 % of
+    # the rows at width 128 with 8 hidden layers). 98 % of the rows must be inside the elementwise bar in every element,
+    # and the whole matrix within 2e-2 in the Frobenius norm (1.2e-2 measured).
+    dXh = dXs.float().cpu().numpy()
+    diff, bar = np.abs(dXh - rdX), 5e-4 * np.abs(rdX).max() + 5e-3 * np.abs(rdX)
+    assert (diff <= bar).all(axis=1).mean() >= 0.98
+    assert np.linalg.norm((dXh - rdX).ravel()) <= 2e-2 * np.linalg.norm(rdX.ravel())

@@ -110,6 +110,96 @@ __global__ void __launch_bounds__(THREADS, (THREADS == 512 && W <= 64) ? 4 : 1)
 }
 
 // ------------------------------------------------------------------------------------------
+// Forward for networks whose weights do not fit LDS (width 128 with more than four matrices): the
+// matrices stream through a double-buffered LDS slot, one layer at a time, for a round of 512 batch
+// rows (8 waves x 2 tiles of 32 rows). While a layer is being computed from one slot, every thread
+// carries its 64-byte share of the next matrix from L2 to the other slot; one barrier per layer. A
+// wave feeds each weight fragment it reads from LDS to two MFMAs (its two tiles), which halves the
+// LDS traffic per flop; reading the fragments from global memory instead (as the in-LDS kernel
+// does when it has no room) is bound by the vector cache at 16 % of the MFMA peak.
+// ------------------------------------------------------------------------------------------
+constexpr int kStreamThreads = 512;
+constexpr int kStreamTiles = 2;
+
+template <typename T, int W, int ACT, bool STORE_INTERM>
+__global__ void __launch_bounds__(kStreamThreads, 1)
+    mlp_forward_stream_kernel(const typename Storage<T>::vec8 *__restrict__ wprep, const T *__restrict__ x, T *__restrict__ out,
+                              int n_mats, int out_act, long long M) {
+    typedef Tile<T, W> TL;
+    typedef typename Storage<T>::vec8 vec8;
+    constexpr int NK = TL::NK, NI = TL::NI, R = kStreamTiles;
+    constexpr int per_mat = NI * NK * kWaveSize;         // 16-byte fragments per matrix
+    constexpr int SHARE = per_mat / kStreamThreads;      // fragments a thread carries per matrix
+    static_assert(per_mat % kStreamThreads == 0, "matrix does not split evenly over the workgroup");
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+    vec8 *lds = reinterpret_cast<vec8 *>(smem_raw); // slot s starts at lds + s * per_mat
+
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int j = lane & 31, h = lane >> 5;
+    constexpr int ROUND = (kStreamThreads / 64) * R * 32;
+    const long long n_rounds = (M + ROUND - 1) / ROUND;
+
+    vec8 st[SHARE];
+#pragma unroll
+    for (int i = 0; i < SHARE; ++i) lds[threadIdx.x + kStreamThreads * i] = wprep[threadIdx.x + kStreamThreads * i];
+    int b = 0; // slot that holds the matrix of the layer about to run
+
+    for (long long r = blockIdx.x; r < n_rounds; r += gridDim.x) {
+        long long row[R];
+        bool valid[R];
+        vec8 cur[R][NK];
+#pragma unroll
+        for (int t = 0; t < R; ++t) {
+            row[t] = r * ROUND + (wave * R + t) * 32 + j;
+            valid[t] = row[t] < M;
+            TL::load(cur[t], x, row[t], h, valid[t]);
+            if (STORE_INTERM) TL::store(cur[t], out, row[t], h, valid[t]);
+        }
+        const bool more_rounds = r + gridDim.x < n_rounds;
+        for (int l = 0; l < n_mats; ++l) {
+            __syncthreads(); // the matrix of layer l is in slot b; nobody reads the other slot any more
+            const bool last = l + 1 == n_mats;
+            const bool stage = !last || more_rounds;
+            const vec8 *next = wprep + (size_t)(last ? 0 : l + 1) * per_mat;
+            if (stage) {
+#pragma unroll
+                for (int i = 0; i < SHARE; ++i) st[i] = next[threadIdx.x + kStreamThreads * i];
+            }
+            f32x16 acc[R][NI];
+#pragma unroll
+            for (int t = 0; t < R; ++t)
+#pragma unroll
+                for (int a = 0; a < NI; ++a) acc[t][a] = f32x16{};
+            const vec8 *w = lds + b * per_mat + lane;
+#pragma unroll
+            for (int kb = 0; kb < NK; ++kb) {
+#pragma unroll
+                for (int a = 0; a < NI; ++a) {
+                    const vec8 frag = w[(a * NK + kb) * kWaveSize];
+#pragma unroll
+                    for (int t = 0; t < R; ++t) acc[t][a] = Storage<T>::mfma(frag, cur[t][kb], acc[t][a]);
+                }
+            }
+            if (stage) {
+#pragma unroll
+                for (int i = 0; i < SHARE; ++i) lds[(b ^ 1) * per_mat + threadIdx.x + kStreamThreads * i] = st[i];
+            }
+#pragma unroll
+            for (int t = 0; t < R; ++t) {
+                if (!last) {
+                    TL::template repack<ACT>(cur[t], acc[t]);
+                    if (STORE_INTERM) TL::store(cur[t], out + (size_t)(l + 1) * M * W, row[t], h, valid[t]);
+                } else {
+                    TL::repack_rt(cur[t], acc[t], out_act);
+                    TL::store(cur[t], STORE_INTERM ? out + (size_t)n_mats * M * W : out, row[t], h, valid[t]);
+                }
+            }
+            b ^= 1;
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------
 // Backward: delta propagation (include/network/kernel_esimd.h:186-227)
 // ------------------------------------------------------------------------------------------
 template <typename T, int W, bool W_IN_LDS>
@@ -345,6 +435,20 @@ static int launch_forward_v(const tnn_mlp_desc *d, const void *wprep, const void
     const DeviceInfo &di = device_info();
     if (!di.ok) return fail(TNN_ERR_HIP, "no usable HIP device");
     const bool in_lds = wbytes <= kLdsBudget;
+    if constexpr (W == 128) {
+        if (!in_lds) { // stream the matrices through LDS, one layer at a time
+            constexpr size_t lds = 2 * (size_t)Tile<T, W>::NI * Tile<T, W>::NK * kWaveSize * sizeof(vec8);
+            constexpr long long round = (kStreamThreads / 64) * kStreamTiles * 32;
+            long long g = ((long long)M + round - 1) / round;
+            if (g > di.n_cu) g = di.n_cu;
+            auto k = mlp_forward_stream_kernel<T, W, ACT, STORE_INTERM>;
+            if (hipFuncSetAttribute(reinterpret_cast<const void *>(k), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+                return fail(TNN_ERR_HIP, "cannot reserve %zu bytes of LDS", lds);
+            TNN_LAUNCH(k, dim3((unsigned)g), dim3(kStreamThreads), lds, s, (const vec8 *)wprep, (const T *)x, (T *)out, n_mats,
+                       d->output_activation, (long long)M);
+            return check_launch("mlp_forward_stream_kernel");
+        }
+    }
     const long long n_tiles = ((long long)M + 31) / 32;
     const int waves = THREADS / 64;
     long long blocks = (n_tiles + waves - 1) / waves;

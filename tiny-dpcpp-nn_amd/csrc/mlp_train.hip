@@ -14,7 +14,10 @@ template <int W> static FusedPlan plan_w(int n_mats, size_t M, int n_cu) {
     p.supported = n_mats >= 2 && n_mats <= max_mats && p.lds <= kMaxLds;
     const long long n_tiles = ((long long)M + 31) / 32;
     long long g = (n_tiles + S::WAVES - 1) / S::WAVES;
-    if (g > n_cu) g = n_cu;
+    // The workspace is sized for two workgroups per CU where the shallow narrow networks leave registers for them; the
+    // launch asks the runtime how many actually fit and may use fewer.
+    const int per_cu = (W <= 32 && n_mats <= 3) ? 2 : 1;
+    if (g > (long long)n_cu * per_cu) g = (long long)n_cu * per_cu;
     if (g < 1) g = 1;
     p.grid = (int)g;
     p.partial_bytes = (size_t)p.grid * n_mats * W * W * sizeof(float);

@@ -264,6 +264,31 @@ int tnn_grid_backward(const tnn_grid_desc *desc, const float *d_x, const void *d
  * d_indices: M x n_levels x 2^n_dims uint32. */
 int tnn_grid_indices(const tnn_grid_desc *desc, const float *d_x, uint32_t *d_indices, size_t M, tnn_stream_t stream);
 
+/* ------------------------------------------------------------------------------------------
+ * Encodings without parameters. Rows are M x padded_width of out_dtype; the columns beyond the encoding's own
+ * width are filled with ONES (the grid pads with zeros). Inputs are M x n_dims fp32, row-major.
+ * ------------------------------------------------------------------------------------------ */
+
+/* IdentityEncoding::forward_impl (include/encodings/identity.h:33-79): out = x * scale + offset. */
+int tnn_identity_forward(const float *d_x, uint32_t n_dims, float scale, float offset, void *d_out, int out_dtype,
+                         uint32_t padded_width, size_t M, tnn_stream_t stream);
+
+/* FrequencyEncoding::forward_impl (include/encodings/frequency.h:30-90): column j of a row is
+ * sin(x[j / (2 n_f)] * 2^((j / 2) % n_f) * pi + (j % 2) * pi / 2). d_dy_dx: NULL, or M x (n_dims * n_f * 2) fp32
+ * that receives the derivative of every output column (the reference's ForwardContext::dy_dx, :41-47,82-84). */
+int tnn_frequency_forward(const float *d_x, uint32_t n_dims, uint32_t n_frequencies, void *d_out, int out_dtype,
+                          uint32_t padded_width, float *d_dy_dx, size_t M, tnn_stream_t stream);
+/* FrequencyEncoding::backward_impl (include/encodings/frequency.h:92-131): dL/dx = sum over a feature's columns of
+ * dL/dy * dy/dx. d_dLdx: M x n_dims fp32. */
+int tnn_frequency_backward(const void *d_dLdy, int dy_dtype, uint32_t padded_width, const float *d_dy_dx, uint32_t n_dims,
+                           uint32_t n_frequencies, float *d_dLdx, size_t M, tnn_stream_t stream);
+
+/* SphericalHarmonicsEncoding::forward_impl with sh_enc (include/encodings/spherical_harmonics.h:38-72,
+ * include/common/common_device.h:33-206): the degree^2 real spherical harmonics of bands 0 .. degree-1 at the
+ * direction 2x - 1 (x: M x 3). degree 1 .. 8. */
+int tnn_sh_forward(const float *d_x, uint32_t degree, void *d_out, int out_dtype, uint32_t padded_width, size_t M,
+                   tnn_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -22,10 +22,17 @@
  *   adam_step ................... torch.optim.Adam on CPU
  *   grid_* ...................... golden vector test/doctest_encodings.cpp:234-285, zero-gradient
  *                                 case :286-341, brute-force dense indexing, adjoint identity
+ *   identity / frequency ........ closed forms of test/doctest_encodings.cpp:156-195,486-584
+ *   sh_forward .................. golden rows of test/python/test_encodings.py:389-573 (degree 4), the degree-1 vector of
+ *                                 test/doctest_encodings.cpp:197-232, the reference's explicit expressions of bands 0-3
+ *                                 (sh_explicit16) and of single members of bands 4-7, orthonormality on the sphere
  *   default table init / Xavier init of the reference: parity unpinned (unseeded / closed-source
  *   generators in the reference); not restated here.
  */
 #include <math.h>
+#ifndef M_PI
+#define M_PI 3.14159265358979323846 /* strict C99 leaves it out of math.h */
+#endif
 #include <stdint.h>
 #include <stdlib.h>
 #include <string.h>
@@ -659,5 +666,124 @@ TNN_ORACLE_API int tnn_oracle_grid_backward(int n_dims, int n_levels, int F, int
     }
     for (size_t p = 0; p < n_params; ++p) grad_table[p] = (float)acc[p];
     free(acc);
+    return 0;
+}
+
+/* ------------------------------------------------------------------------- */
+/* Encodings without parameters                                               */
+/* ------------------------------------------------------------------------- */
+
+/* include/encodings/identity.h:61-75 : in * scale + offset, ones beyond the encoded columns */
+TNN_ORACLE_API void tnn_oracle_identity_forward(const float *x, int n_dims, float scale, float offset, size_t M, float *out,
+                                                int padded_width) {
+    for (size_t i = 0; i < M; ++i)
+        for (int j = 0; j < padded_width; ++j)
+            out[i * padded_width + j] = j >= n_dims ? 1.0f : x[i * n_dims + j] * scale + offset;
+}
+
+/* include/encodings/frequency.h:62-86 : the argument is float * size_t (a float product), times M_PI and plus the
+ * phase shift in double, rounded to float once; sine in float. dy_dx (may be NULL): M x (n_dims * n_freq * 2). */
+TNN_ORACLE_API void tnn_oracle_frequency_forward(const float *x, int n_dims, int n_freq, size_t M, float *out, int padded_width,
+                                                 float *dy_dx) {
+    const int width = n_dims * n_freq * 2;
+    for (size_t i = 0; i < M; ++i)
+        for (int j = 0; j < padded_width; ++j) {
+            if (j >= width) {
+                out[i * padded_width + j] = 1.0f;
+                continue;
+            }
+            const int feature = j / (n_freq * 2), log2_frequency = (j / 2) % n_freq;
+            const float phase_shift = (float)((j % 2) * (M_PI / 2.0f));
+            const float scaled = x[i * n_dims + feature] * (float)((size_t)1 << log2_frequency);
+            const float arg = (float)((double)scaled * M_PI + (double)phase_shift);
+            out[i * padded_width + j] = sinf(arg);
+            if (dy_dx) dy_dx[i * width + j] = (float)((double)(float)((size_t)1 << log2_frequency) * M_PI * (double)cosf(arg));
+        }
+}
+
+/* include/encodings/frequency.h:108-126 */
+TNN_ORACLE_API void tnn_oracle_frequency_backward(const float *dLdy, int padded_width, const float *dy_dx, int n_dims, int n_freq,
+                                                  size_t M, float *dLdx) {
+    const int per_input = n_freq * 2, width = n_dims * per_input;
+    for (size_t i = 0; i < M; ++i)
+        for (int j = 0; j < n_dims; ++j) {
+            double r = 0.0;
+            for (int k = 0; k < per_input; ++k)
+                r += (double)dLdy[i * padded_width + j * per_input + k] * (double)dy_dx[i * width + j * per_input + k];
+            dLdx[i * n_dims + j] = (float)r;
+        }
+}
+
+/* The first 16 real spherical harmonics as the reference spells them out (include/common/common_device.h:47-70; the
+ * constants are the closed forms given in its comments). Arguments are the direction itself (no 2x-1 here). */
+TNN_ORACLE_API void tnn_oracle_sh_explicit16(double x, double y, double z, double *o) {
+    const double sp = sqrt(M_PI);
+    const double xy = x * y, xz = x * z, yz = y * z, x2 = x * x, y2 = y * y, z2 = z * z;
+    o[0] = 1.0 / (2.0 * sp);
+    o[1] = -sqrt(3.0) * y / (2.0 * sp);
+    o[2] = sqrt(3.0) * z / (2.0 * sp);
+    o[3] = -sqrt(3.0) * x / (2.0 * sp);
+    o[4] = sqrt(15.0) * xy / (2.0 * sp);
+    o[5] = -sqrt(15.0) * yz / (2.0 * sp);
+    o[6] = sqrt(5.0) * (3.0 * z2 - 1.0) / (4.0 * sp);
+    o[7] = -sqrt(15.0) * xz / (2.0 * sp);
+    o[8] = sqrt(15.0) * (x2 - y2) / (4.0 * sp);
+    o[9] = sqrt(70.0) * y * (-3.0 * x2 + y2) / (8.0 * sp);
+    o[10] = sqrt(105.0) * xy * z / (2.0 * sp);
+    o[11] = sqrt(42.0) * y * (1.0 - 5.0 * z2) / (8.0 * sp);
+    o[12] = sqrt(7.0) * z * (5.0 * z2 - 3.0) / (4.0 * sp);
+    o[13] = sqrt(42.0) * x * (1.0 - 5.0 * z2) / (8.0 * sp);
+    o[14] = sqrt(105.0) * z * (x2 - y2) / (4.0 * sp);
+    o[15] = sqrt(70.0) * x * (-x2 + 3.0 * y2) / (8.0 * sp);
+}
+
+/* include/encodings/spherical_harmonics.h:55-70 with sh_enc (include/common/common_device.h:33-206). The reference's
+ * unrolled expressions were generated from the recurrences of appendix A1 of P.-P. Sloan, "Stupid Spherical Harmonics
+ * (SH) Tricks" (common_device.h:43-46); this restates those recurrences, in double:
+ *   Y(l, m) = K(l,|m|) * P(l,|m|)(z) * { sqrt2 Re (x+iy)^m | 1 | sqrt2 Im (x+iy)^|m| },  index l^2 + l + m,
+ *   P(m,m) = (-1)^m (2m-1)!!,  P(m+1,m) = (2m+1) z P(m,m),  P(l,m) = ((2l-1) z P(l-1,m) - (l+m-1) P(l-2,m)) / (l-m).
+ * Input x in [0,1]^3 is mapped to the direction 2x-1; columns beyond degree^2 are ones. */
+TNN_ORACLE_API int tnn_oracle_sh_forward(int degree, const float *xin, size_t M, float *out, int padded_width) {
+    if (degree < 1 || degree > 8 || padded_width < degree * degree) return -1;
+    for (size_t i = 0; i < M; ++i) {
+        /* the reference forms 2x-1 in float */
+        const double x = (double)(xin[i * 3 + 0] * 2.f - 1.f), y = (double)(xin[i * 3 + 1] * 2.f - 1.f),
+                     z = (double)(xin[i * 3 + 2] * 2.f - 1.f);
+        float *row = out + i * padded_width;
+        double cm = 1.0, sm = 0.0, pmm = 1.0;
+        for (int m = 0; m < degree; ++m) {
+            if (m > 0) {
+                const double cn = cm * x - sm * y;
+                sm = cm * y + sm * x;
+                cm = cn;
+                pmm *= -(double)(2 * m - 1);
+            }
+            double p2 = 0.0, p1 = pmm;
+            for (int l = m; l < degree; ++l) {
+                double p;
+                if (l == m) {
+                    p = pmm;
+                } else if (l == m + 1) {
+                    p = (2 * m + 1) * z * pmm;
+                } else {
+                    p = ((2 * l - 1) * z * p1 - (l + m - 1) * p2) / (l - m);
+                }
+                if (l > m) {
+                    p2 = p1;
+                    p1 = p;
+                }
+                double ratio = 1.0;
+                for (int t = l - m + 1; t <= l + m; ++t) ratio /= (double)t;
+                const double k = sqrt((2.0 * l + 1.0) / (4.0 * M_PI) * ratio) * (m > 0 ? sqrt(2.0) : 1.0);
+                if (m == 0) {
+                    row[l * l + l] = (float)(k * p);
+                } else {
+                    row[l * l + l + m] = (float)(k * p * cm);
+                    row[l * l + l - m] = (float)(k * p * sm);
+                }
+            }
+        }
+        for (int j = degree * degree; j < padded_width; ++j) row[j] = 1.0f;
+    }
     return 0;
 }

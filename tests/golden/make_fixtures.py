@@ -64,6 +64,20 @@ def main():
         open(os.path.join(HERE, "packed_coords.json"), "w"),
     )
 
+    # test/python/test_encodings.py:377-573 : spherical harmonics of degree 4 at the input (1, 1, 1) (ten equal rows)
+    txt = open(os.path.join(REF, "test/python/test_encodings.py")).read()
+    s = txt.index("def test_spherical():")
+    vals = numbers_between(txt[s:], "spherical_output = torch.Tensor(", ").to(")
+    assert len(vals) == 160 and vals[:16] == vals[16:32]
+    json.dump(
+        {
+            "source": "test/python/test_encodings.py:377-573",
+            "degree": 4, "input": [1.0, 1.0, 1.0], "n_rows": 10, "atol": 1.0e-3,
+            "expected_row": vals[:16],
+        },
+        open(os.path.join(HERE, "spherical_harmonics_degree4.json"), "w"),
+    )
+
 
 if __name__ == "__main__":
     main()

@@ -146,6 +146,32 @@ class Harness:
         _lib.check(self.lib.tnn_grid_backward(ctypes.byref(d), ptr(x_t), ptr(dLdy_t), dy_dtype, pw, ptr(grad_t), int(overwrite), M, self.stream()))
         return grad_t
 
+    # ------------------------------------------------------------------------------
+    def identity_forward(self, x_t, scale, offset, padded_width, out_dtype=FP32):
+        M, D = x_t.shape
+        out = torch.full((M, padded_width), float("nan"), dtype=TORCH_DT[out_dtype], device=self.dev)
+        _lib.check(self.lib.tnn_identity_forward(ptr(x_t), D, scale, offset, ptr(out), out_dtype, padded_width, M, self.stream()))
+        return out
+
+    def frequency_forward(self, x_t, n_freq, padded_width, out_dtype=FP32, want_dy_dx=False):
+        M, D = x_t.shape
+        out = torch.full((M, padded_width), float("nan"), dtype=TORCH_DT[out_dtype], device=self.dev)
+        dy = torch.full((M, D * n_freq * 2), float("nan"), dtype=torch.float32, device=self.dev) if want_dy_dx else None
+        _lib.check(self.lib.tnn_frequency_forward(ptr(x_t), D, n_freq, ptr(out), out_dtype, padded_width, ptr(dy), M, self.stream()))
+        return (out, dy) if want_dy_dx else out
+
+    def frequency_backward(self, dLdy_t, dy_dtype, dy_dx_t, n_dims, n_freq):
+        M, pw = dLdy_t.shape
+        out = torch.full((M, n_dims), float("nan"), dtype=torch.float32, device=self.dev)
+        _lib.check(self.lib.tnn_frequency_backward(ptr(dLdy_t), dy_dtype, pw, ptr(dy_dx_t), n_dims, n_freq, ptr(out), M, self.stream()))
+        return out
+
+    def sh_forward(self, x_t, degree, padded_width, out_dtype=FP32):
+        M = x_t.shape[0]
+        out = torch.full((M, padded_width), float("nan"), dtype=TORCH_DT[out_dtype], device=self.dev)
+        _lib.check(self.lib.tnn_sh_forward(ptr(x_t), degree, ptr(out), out_dtype, padded_width, M, self.stream()))
+        return out
+
     def grid_indices(self, d, x_t):
         M = x_t.shape[0]
         out = torch.empty((M, d.n_levels, 1 << d.n_dims), dtype=torch.int32, device=self.dev)

@@ -48,6 +48,11 @@ class Oracle:
                                               c_size_t, c_void_p, c_int]
         L.tnn_oracle_grid_backward.argtypes = [c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_void_p, c_void_p,
                                                c_size_t, c_int, c_void_p]
+        L.tnn_oracle_identity_forward.argtypes = [c_void_p, c_int, c_float, c_float, c_size_t, c_void_p, c_int]
+        L.tnn_oracle_frequency_forward.argtypes = [c_void_p, c_int, c_int, c_size_t, c_void_p, c_int, c_void_p]
+        L.tnn_oracle_frequency_backward.argtypes = [c_void_p, c_int, c_void_p, c_int, c_int, c_size_t, c_void_p]
+        L.tnn_oracle_sh_explicit16.argtypes = [ctypes.c_double] * 3 + [c_void_p]
+        L.tnn_oracle_sh_forward.argtypes = [c_int, c_void_p, c_size_t, c_void_p, c_int]
         L.tnn_oracle_num_threads.restype = c_int
         L.tnn_oracle_set_num_threads.argtypes = [c_int]
 
@@ -192,3 +197,37 @@ class Oracle:
         if rc:
             raise ValueError("grid_backward")
         return grad
+
+    # --- encodings without parameters -------------------------------------------------------
+    def identity_forward(self, x, scale, offset, padded_width):
+        x = _f32(x)
+        out = np.empty((x.shape[0], padded_width), np.float32)
+        self.L.tnn_oracle_identity_forward(_p(x), x.shape[1], scale, offset, x.shape[0], _p(out), padded_width)
+        return out
+
+    def frequency_forward(self, x, n_freq, padded_width, want_dy_dx=False):
+        x = _f32(x)
+        M, D = x.shape
+        out = np.empty((M, padded_width), np.float32)
+        dy = np.empty((M, D * n_freq * 2), np.float32) if want_dy_dx else None
+        self.L.tnn_oracle_frequency_forward(_p(x), D, n_freq, M, _p(out), padded_width, _p(dy) if want_dy_dx else None)
+        return (out, dy) if want_dy_dx else out
+
+    def frequency_backward(self, dLdy, dy_dx, n_dims, n_freq):
+        dLdy, dy_dx = _f32(dLdy), _f32(dy_dx)
+        M = dLdy.shape[0]
+        out = np.empty((M, n_dims), np.float32)
+        self.L.tnn_oracle_frequency_backward(_p(dLdy), dLdy.shape[1], _p(dy_dx), n_dims, n_freq, M, _p(out))
+        return out
+
+    def sh_explicit16(self, x, y, z):
+        out = np.empty(16, np.float64)
+        self.L.tnn_oracle_sh_explicit16(float(x), float(y), float(z), _p(out))
+        return out
+
+    def sh_forward(self, degree, x, padded_width):
+        x = _f32(x)
+        out = np.full((x.shape[0], padded_width), np.nan, np.float32)
+        if self.L.tnn_oracle_sh_forward(degree, _p(x), x.shape[0], _p(out), padded_width):
+            raise ValueError("sh_forward")
+        return out

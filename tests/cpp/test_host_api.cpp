@@ -24,6 +24,10 @@ void tnn_oracle_l2_loss(int dtype, const float *pred, const float *target, size_
 int tnn_oracle_grid_forward(int n_dims, int n_levels, int F, int log2_hashmap_size, int base_resolution, float per_level_scale,
                             int grid_type, int hash_type, int interp, const float *table, const float *x, size_t M, float *out,
                             int padded_width);
+void tnn_oracle_identity_forward(const float *x, int n_dims, float scale, float offset, size_t M, float *out, int padded_width);
+void tnn_oracle_frequency_forward(const float *x, int n_dims, int n_freq, size_t M, float *out, int padded_width, float *dy_dx);
+void tnn_oracle_frequency_backward(const float *dLdy, int padded_width, const float *dy_dx, int n_dims, int n_freq, size_t M, float *dLdx);
+int tnn_oracle_sh_forward(int degree, const float *xin, size_t M, float *out, int padded_width);
 int tnn_oracle_grid_backward(int n_dims, int n_levels, int F, int log2_hashmap_size, int base_resolution, float per_level_scale,
                              int grid_type, int hash_type, int interp, const float *x, const float *dLdy, size_t M, int padded_width,
                              float *grad_table);
@@ -469,6 +473,88 @@ static void test_grid(const char *config_text, uint32_t padded_width, size_t M) 
     CHECK(enc->forward_impl(xd.GetView(), nullptr) == nullptr);
 }
 
+static double max_abs_diff(const std::vector<float> &a, const std::vector<float> &b) {
+    double d = 0;
+    for (size_t i = 0; i < a.size(); ++i) d = std::max(d, (double)std::fabs(a[i] - b[i]));
+    return d;
+}
+
+// test/doctest_encodings.cpp:156-232,346-584 of the reference, plus the oracle on seeded inputs
+static void test_parameter_free_encodings() {
+    std::printf(" identity / frequency / spherical harmonics\n");
+    tnn::queue q;
+    const size_t M = 500;
+    std::vector<float> x = uniform(M * 3, 0.f, 1.f, 21);
+    DeviceMatrix<float> xd(M, 3, q);
+    xd.copy_from_host(x);
+    {
+        auto enc = create_encoding<float>(json::parse(R"({"otype": "Identity", "n_dims_to_encode": 3, "scale": 1.5, "offset": 0.25})"), q, 8u);
+        CHECK(enc->get_input_width() == 3 && enc->get_output_width() == 3 && enc->get_padded_output_width() == 8 && enc->get_n_params() == 0 &&
+              enc->get_params() == nullptr && enc->get_n_to_pad() == 5);
+        DeviceMatrix<float> out(M, 8, q);
+        DeviceMatrixView<float> v = out.GetView();
+        CHECK(enc->forward_impl(xd.GetView(), &v) != nullptr);
+        std::vector<float> ref(M * 8);
+        tnn_oracle_identity_forward(x.data(), 3, 1.5f, 0.25f, M, ref.data(), 8);
+        CHECK(out.copy_to_host() == ref);
+        Context ctx;
+        CHECK(throws<std::logic_error>([&] { enc->backward_impl(ctx, xd.GetView(), v); }, "Not yet implemented"));
+        DeviceMatrix<float> bad(M, 9, q);
+        DeviceMatrixView<float> bv = bad.GetView();
+        CHECK(throws<std::invalid_argument>([&] { enc->forward_impl(xd.GetView(), &bv); }, "padded output width"));
+        CHECK(throws<std::invalid_argument>([&] { create_encoding<float>(json::parse(R"({"otype": "Identity", "n_dims_to_encode": 3, "scale": 1.0})"), q); },
+                                            "Config misses offset"));
+    }
+    {
+        const json cfg = json::parse(R"({"otype": "Frequency", "n_dims_to_encode": 3, "n_frequencies": 6})");
+        auto enc = create_encoding<float>(cfg, q, 48u);
+        CHECK(enc->get_output_width() == 36 && enc->get_padded_output_width() == 48);
+        CHECK(create_encoding<float>(cfg, q)->get_padded_output_width() == 36);
+        DeviceMatrix<float> out(M, 48, q);
+        DeviceMatrixView<float> v = out.GetView();
+        std::unique_ptr<Context> ctx = enc->forward_impl(xd.GetView(), &v, false, true);
+        std::vector<float> ref(M * 48), dy(M * 36);
+        tnn_oracle_frequency_forward(x.data(), 3, 6, M, ref.data(), 48, dy.data());
+        CHECK(max_abs_diff(out.copy_to_host(), ref) <= 2e-6);
+        std::vector<float> g = uniform(M * 48, -1.f, 1.f, 22), dref(M * 3);
+        DeviceMatrix<float> gd(M, 48, q), dx(M, 3, q);
+        gd.copy_from_host(g);
+        enc->backward_impl(*ctx, xd.GetView(), gd.GetView(), nullptr, &dx);
+        const std::vector<float> dxh = dx.copy_to_host();
+        // the oracle gets its own derivatives; cos of arguments up to 32 pi differs by ulps between host and device
+        tnn_oracle_frequency_backward(g.data(), 48, dy.data(), 3, 6, M, dref.data());
+        CHECK(max_norm_rel(dxh, dref) <= 1e-4);
+        std::unique_ptr<Context> plain = enc->forward_impl(xd.GetView(), &v);
+        CHECK(throws<std::bad_cast>([&] { enc->backward_impl(*plain, xd.GetView(), gd.GetView(), nullptr, &dx); }));
+        // creation cases of the reference's doctest
+        CHECK(throws<std::invalid_argument>([&] { create_encoding<float>(json::parse(R"({"otype": "Frequency", "n_dims_to_encode": 1})"), q); }));
+        CHECK(throws<std::invalid_argument>([&] { create_encoding<float>(json::parse(R"({"otype": "Frequency", "n_dims_to_encode": 1, "n_frequencies": 0})"), q); }));
+        CHECK(throws<std::invalid_argument>([&] { create_encoding<float>(json::parse(R"({"otype": "Frequency", "n_dims_to_encode": 1, "n_frequencies": -1})"), q); }));
+        CHECK(throws<std::invalid_argument>([&] { create_encoding<float>(json::parse(R"({"otype": "Frequency", "n_dims_to_encode": 0, "n_frequencies": 1})"), q); }));
+        CHECK(throws<std::invalid_argument>([&] { create_encoding<float>(json::parse(R"({"otype": "Frequency", "n_dims_to_encode": 1, "n_frequencies": 1})"), q, 1u); }));
+        CHECK(create_encoding<float>(json::parse(R"({"otype": "Frequency", "n_dims_to_encode": 1, "n_frequencies": 1})"), q, 2u) != nullptr);
+    }
+    {
+        auto enc = create_encoding<float>(json::parse(R"({"otype": "SphericalHarmonics", "n_dims_to_encode": 3, "degree": 4})"), q, 32u);
+        CHECK(enc->get_output_width() == 16 && enc->get_padded_output_width() == 32);
+        DeviceMatrix<float> out(M, 32, q);
+        DeviceMatrixView<float> v = out.GetView();
+        enc->forward_impl(xd.GetView(), &v);
+        q.wait();
+        std::vector<float> ref(M * 32);
+        CHECK(tnn_oracle_sh_forward(4, x.data(), M, ref.data(), 32) == 0);
+        CHECK(max_abs_diff(out.copy_to_host(), ref) <= 2e-5);
+        Context ctx;
+        CHECK(throws<std::logic_error>([&] { enc->backward_impl(ctx, xd.GetView(), v); }, "not yet implemented"));
+        CHECK(throws<std::runtime_error>([&] { create_encoding<float>(json::parse(R"({"otype": "SphericalHarmonics", "n_dims_to_encode": 2, "degree": 4})"), q); },
+                                         "3D directions"));
+        CHECK(throws<std::runtime_error>([&] { create_encoding<float>(json::parse(R"({"otype": "SphericalHarmonics", "n_dims_to_encode": 3, "degree": 9})"), q); },
+                                         "degree"));
+        CHECK(throws<std::invalid_argument>([&] { create_encoding<float>(json::parse(R"({"otype": "SphericalHarmonics", "n_dims_to_encode": 3})"), q); },
+                                            "Config misses degree"));
+    }
+}
+
 static void test_encoding_config_errors() {
     std::printf(" encoding configuration errors\n");
     tnn::queue q;
@@ -516,6 +602,7 @@ int main(int argc, char **argv) {
                       "base_resolution": 8, "interpolation": "Smoothstep"})", 16, 777);
         test_grid(R"({"otype": "HashGrid", "type": "Tiled", "n_dims_to_encode": 3, "n_features": 6, "n_features_per_level": 1,
                       "base_resolution": 5, "per_level_scale": 2.0, "interpolation": "Nearest"})", 16, 256);
+        test_parameter_free_encodings();
         test_encoding_config_errors();
     }
     std::printf("%d checks, %d failed\n", g_checks, g_failed);

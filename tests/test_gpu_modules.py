@@ -315,3 +315,47 @@ def test_network_with_input_encoding_trains(tcnn, dtype):
     assert float(((out.float() - target(xy)) ** 2).mean()) < 0.5 * losses[0]
     with pytest.raises(RuntimeError, match="Not implemented"):
         model.get_params()
+
+
+def test_parameter_free_encodings_through_the_package(tcnn, oracle):
+    """test/python/test_encodings.py:377-630 of the reference: spherical harmonics (golden rows), identity, padding, frequency."""
+    import json
+    import math
+    import os
+
+    ones = torch.ones((10, 3), device=DEVICE)
+    sh = tcnn.Encoding(n_input_dims=3, encoding_config={"otype": "SphericalHarmonics", "degree": 4})
+    assert sh.n_output_dims == 16 and not sh.params.requires_grad
+    fx = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "spherical_harmonics_degree4.json")))
+    out = sh(ones)
+    assert out.shape == (10, 16) and out.dtype == torch.float32
+    assert torch.all(torch.isclose(out.cpu(), torch.tensor(fx["expected_row"]).expand(10, 16), atol=fx["atol"]))
+
+    ident = tcnn.Encoding(n_input_dims=3, encoding_config={"otype": "Identity", "scale": 1.0, "offset": 0.0})
+    assert torch.all(torch.isclose(ident(ones), ones))
+    wide = tcnn.Encoding(n_input_dims=3, encoding_config={"otype": "Identity", "scale": 1.0, "offset": 0.0}, n_output_dims=5346)
+    y = wide(torch.rand((13, 3), device=DEVICE))            # a batch that is not a multiple of 8
+    assert wide.n_output_dims == 5346 and y.shape == (13, 5346) and bool((y[:, 3:] == 1).all())
+
+    freq = tcnn.Encoding(n_input_dims=1, encoding_config={"otype": "Frequency", "n_frequencies": 1.0})
+    v = 1.234
+    out = freq(torch.ones(1, 1, device=DEVICE) * v)
+    assert torch.allclose(out.cpu(), torch.tensor([[math.sin(math.pi * v), math.cos(math.pi * v)]]), atol=1e-4)
+
+    x = torch.rand((100, 3), device=DEVICE)
+    f2 = tcnn.Encoding(n_input_dims=3, encoding_config={"otype": "Frequency", "n_frequencies": 4}, n_output_dims=32)
+    np.testing.assert_allclose(f2(x).cpu().numpy(), oracle.frequency_forward(x.cpu().numpy(), 4, 32), atol=2e-6)
+    with pytest.raises((RuntimeError, ValueError), match="Config misses"):
+        tcnn.Encoding(n_input_dims=3, encoding_config={"otype": "Identity", "scale": 1.0})
+    with pytest.raises(RuntimeError, match="Network has no parameters"):
+        ident.set_params(torch.zeros(3, device=DEVICE))
+
+
+def test_nerf_style_directional_network(tcnn):
+    """test/python/test_nerf_settings.py:80-86 of the reference: spherical harmonics of degree 4 feeding a network."""
+    model = tcnn.NetworkWithInputEncoding(3, 3, net_config(64, 2), {"otype": "SphericalHarmonics", "degree": 4}, dtype=torch.bfloat16)
+    x = torch.rand((1000, 3), device=DEVICE)
+    y = model(x)
+    assert y.shape == (1000, 3) and torch.isfinite(y.float()).all()
+    y.float().sum().backward()
+    assert model.network.params.grad is not None and torch.isfinite(model.network.params.grad).all()

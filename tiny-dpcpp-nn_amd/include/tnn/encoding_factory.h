@@ -4,15 +4,65 @@
 
 #include <algorithm>
 #include <iostream>
+#include <limits>
 #include <unordered_set>
 
 #include "encoding.h"
+#include "frequency.h"
 #include "grid.h"
+#include "identity.h"
+#include "spherical_harmonics.h"
 
 template <typename T> class EncodingFactory {
   public:
     virtual ~EncodingFactory() {}
     virtual std::shared_ptr<Encoding<T>> create(const json &config, std::optional<uint32_t> padded_output_width, tnn::queue &Q) const = 0;
+};
+
+template <typename T> class IdentityEncodingFactory : public EncodingFactory<T> {
+  public:
+    std::shared_ptr<Encoding<T>> create(const json &config, std::optional<uint32_t> padded_output_width, tnn::queue &Q) const override {
+        if (!config.contains(EncodingParams::OFFSET)) throw std::invalid_argument("Config misses " + EncodingParams::OFFSET);
+        if (!config.contains(EncodingParams::SCALE)) throw std::invalid_argument("Config misses " + EncodingParams::SCALE);
+        if (!config.contains(EncodingParams::N_DIMS_TO_ENCODE)) throw std::invalid_argument("Config misses " + EncodingParams::N_DIMS_TO_ENCODE);
+        const uint32_t n_dims_to_encode = config[EncodingParams::N_DIMS_TO_ENCODE];
+        const float scale = config[EncodingParams::SCALE];
+        const float offset = config[EncodingParams::OFFSET];
+        return std::make_shared<IdentityEncoding<T>>(n_dims_to_encode, padded_output_width.has_value() ? padded_output_width.value() : n_dims_to_encode,
+                                                     scale, offset, Q);
+    }
+};
+
+template <typename T> class SphericalHarmonicsEncodingFactory : public EncodingFactory<T> {
+  public:
+    std::shared_ptr<Encoding<T>> create(const json &config, std::optional<uint32_t> padded_output_width, tnn::queue &Q) const override {
+        if (!config.contains(EncodingParams::DEGREE)) throw std::invalid_argument("Config misses " + EncodingParams::DEGREE);
+        if (!config.contains(EncodingParams::N_DIMS_TO_ENCODE)) throw std::invalid_argument("Config misses " + EncodingParams::N_DIMS_TO_ENCODE);
+        const uint32_t degree = config[EncodingParams::DEGREE];
+        const uint32_t n_dims_to_encode = config[EncodingParams::N_DIMS_TO_ENCODE];
+        return std::make_shared<SphericalHarmonicsEncoding<T>>(
+            degree, n_dims_to_encode, padded_output_width.has_value() ? padded_output_width.value() : (degree * degree), Q);
+    }
+};
+
+template <typename T> class FrequencyEncodingFactory : public EncodingFactory<T> {
+  public:
+    std::shared_ptr<Encoding<T>> create(const json &config, std::optional<uint32_t> padded_output_width, tnn::queue &Q) const override {
+        if (!config.contains(EncodingParams::N_FREQUENCIES)) throw std::invalid_argument("Config misses " + EncodingParams::N_FREQUENCIES);
+        if (!config.contains(EncodingParams::N_DIMS_TO_ENCODE)) throw std::invalid_argument("Config misses " + EncodingParams::N_DIMS_TO_ENCODE);
+        // negative values are rejected here; the reference lets them wrap to huge unsigned widths, which then fail to allocate
+        const int64_t n_freq = config[EncodingParams::N_FREQUENCIES].template get<int64_t>();
+        const int64_t n_dims = config[EncodingParams::N_DIMS_TO_ENCODE].template get<int64_t>();
+        if (n_freq < 0 || n_dims < 0 || n_freq > 0xffffffffll || n_dims > 0xffffffffll)
+            throw std::invalid_argument("n_frequencies and n_dims_to_encode must be non-negative 32-bit numbers");
+        const uint32_t n_frequencies = (uint32_t)n_freq, n_dims_to_encode = (uint32_t)n_dims;
+        if (n_frequencies == 0) throw std::invalid_argument("Output width cannot be zero");
+        if (std::numeric_limits<uint32_t>::max() / n_frequencies < 2 * n_dims_to_encode)
+            throw std::invalid_argument("n_frequencies * 2 * n_dims_to_encode exceeds uint32_t max");
+        return std::make_shared<FrequencyEncoding<T>>(
+            n_frequencies, n_dims_to_encode,
+            padded_output_width.has_value() ? padded_output_width.value() : 2 * n_frequencies * n_dims_to_encode, Q);
+    }
 };
 
 template <typename T> class GridEncodingFactory : public EncodingFactory<T> {
@@ -45,9 +95,13 @@ std::shared_ptr<Encoding<T>> create_encoding(const json &config, tnn::queue &Q, 
     }
 
     std::unique_ptr<EncodingFactory<T>> factory;
-    if (name == EncodingNames::GRID)
+    if (name == EncodingNames::IDENTITY)
+        factory = std::make_unique<IdentityEncodingFactory<T>>();
+    else if (name == EncodingNames::SPHERICALHARMONICS)
+        factory = std::make_unique<SphericalHarmonicsEncodingFactory<T>>();
+    else if (name == EncodingNames::GRID)
         factory = std::make_unique<GridEncodingFactory<T>>();
     else
-        throw std::invalid_argument("Encoding type " + name + " is not part of this build; only " + EncodingNames::GRID + " is.");
+        factory = std::make_unique<FrequencyEncodingFactory<T>>();
     return factory->create(config, padded_output_width, Q);
 }

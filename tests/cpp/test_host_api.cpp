@@ -364,6 +364,45 @@ static void test_swiftnet_errors() {
     CHECK(f_ok.GetViews().GetElementPointer(3, 1, 2) == f_ok.data() + 3 * 8 * 64 + 64 + 2);
 }
 
+// Trainer with graph recording: every step equals the step run as enqueued (SyclGraph use in include/trainer.h:27-31)
+static void test_trainer_graph() {
+    std::printf(" trainer with HIP graph\n");
+    hipStream_t raw = nullptr;
+    tnn::hip_check(hipStreamCreate(&raw), "hipStreamCreate");
+    {
+        tnn::queue q(raw);
+        typedef tnn::bf16 T;
+        const int W = 64, L = 3;
+        const size_t M = 2048;
+        SwiftNetMLP<T, 64> net(q, W, W, L, Activation::ReLU, Activation::None);
+        Trainer<T> eager(&net, false), recorded(&net, true);
+        DeviceMatrix<T> x(M, W, q), g(M, W, q);
+        DeviceMatrices<T> f1(L + 2, M, W, M, W, M, W, q), b1(L + 1, M, W, M, W, M, W, q), w1(L + 1, W, W, W, W, W, W, q);
+        DeviceMatrices<T> f2(L + 2, M, W, M, W, M, W, q), b2(L + 1, M, W, M, W, M, W, q), w2(L + 1, W, W, W, W, W, W, q);
+        for (int it = 0; it < 4; ++it) {
+            x.copy_from_host(from_float<T>(uniform(M * W, -1.f, 1.f, 100 + it)));
+            g.copy_from_host(from_float<T>(uniform(M * W, -1e-3f, 1e-3f, 200 + it)));
+            eager.training_step(x, w1, g, f1, b1, {});
+            q.wait();
+            f2.fill(T(9.f)).wait();
+            w2.fill(T(9.f)).wait();
+            recorded.training_step(x, w2, g, f2, b2, {});
+            q.wait();
+            CHECK(to_float(f1.copy_to_host()) == to_float(f2.copy_to_host()));
+            CHECK(to_float(b1.copy_to_host()) == to_float(b2.copy_to_host()));
+            CHECK(max_norm_rel(to_float(w1.copy_to_host()), to_float(w2.copy_to_host())) <= 1e-3);
+        }
+        CHECK(recorded.graph().launches() == 3 && eager.graph().launches() == 0); // the first step of a batch size is not recorded
+        // the legacy default stream cannot be recorded: the step then simply runs
+        tnn::queue q0;
+        tinydpcppnn::HipGraph none;
+        { auto guard = none.capture_guard(&q0); }
+        { auto guard = none.capture_guard(nullptr); }
+        CHECK(none.launches() == 0);
+    }
+    tnn::hip_check(hipStreamDestroy(raw), "hipStreamDestroy");
+}
+
 static void test_l2_loss() {
     std::printf(" l2 loss\n");
     tnn::queue q;
@@ -593,6 +632,7 @@ int main(int argc, char **argv) {
         test_swiftnet<tnn::half, 128>(Activation::ReLU, Activation::ReLU, 8, 256, 128, 100, false);
         test_swiftnet<tnn::bf16, 128>(Activation::None, Activation::None, 1, 8, 128, 128, false);
         test_l2_loss();
+        test_trainer_graph();
         std::printf("encodings\n");
         test_grid(R"({"otype": "HashGrid", "n_dims_to_encode": 2, "n_levels": 16, "n_features_per_level": 2, "log2_hashmap_size": 15,
                       "base_resolution": 16, "per_level_scale": 1.5})", 32, 2048);

@@ -359,3 +359,18 @@ def test_nerf_style_directional_network(tcnn):
     assert y.shape == (1000, 3) and torch.isfinite(y.float()).all()
     y.float().sum().backward()
     assert model.network.params.grad is not None and torch.isfinite(model.network.params.grad).all()
+
+
+def test_image_learning_sample(tcnn, monkeypatch):
+    """The sample under tiny-dpcpp-nn_amd/samples (counterpart of the reference's mlp_learning_an_image_pytorch.py) learns its
+    procedural image: 200 steps bring the mean squared error of the rendered image below 1e-3."""
+    import importlib.util
+    import os
+    import sys
+
+    path = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "tiny-dpcpp-nn_amd", "samples", "mlp_learning_an_image.py")
+    spec = importlib.util.spec_from_file_location("mlp_learning_an_image", path)
+    sample = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(sample)
+    monkeypatch.setattr(sys, "argv", ["mlp_learning_an_image.py", "--n_steps", "200"])
+    assert sample.main() < 1e-3

@@ -138,7 +138,6 @@ template <typename T, MatrixLayout _layout = MatrixLayout::RowMajor> class Devic
     }
     template <typename Ts> void copy_from_device(Ts const *const src) {
         tnn::abi_check(tnn_cast(tnn::dtype_of<T>::value, m_data, tnn::dtype_of<Ts>::value, src, n_elements(), m_q.abi()));
-        m_q.wait();
     }
 
     T *data() { return m_data; }

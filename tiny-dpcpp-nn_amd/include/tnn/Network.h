@@ -93,8 +93,9 @@ template <typename T> class Network : public NetworkBase<T> {
             tnn::abi_check(tnn_cast(dtype, m_weightsT_matrices.data(), tnn::dtype_of<Ts>::value, d_weights, n, m_q.abi()));
             tnn::abi_check(tnn_pack_weights(dtype, network_width_, n_hidden_layers_ + 1, m_weightsT_matrices.data(), m_weights_matrices.data(), m_q.abi()));
         }
-        ZeroWeightsPadding(original_input_width_, original_output_width_);
-        TransposeWeights(m_weights_matrices, m_weightsT_matrices);
+        // everything above and below is enqueued on the one in-order stream: no host wait is needed here
+        ZeroWeightsPadding(original_input_width_, original_output_width_, false);
+        TransposeWeights(m_weights_matrices, m_weightsT_matrices, false);
     }
 
     virtual const DeviceMatrices<T> &get_weights_matrices() const { return m_weights_matrices; }
@@ -158,7 +159,7 @@ template <typename T> class Network : public NetworkBase<T> {
 
     /// Zeroes the weights that only see padding: rows of the input matrix at and beyond the one-padded input
     /// width and columns of the output matrix at and beyond the unpadded output width.
-    void ZeroWeightsPadding(const int unpadded_input_width, const int unpadded_output_width) {
+    void ZeroWeightsPadding(const int unpadded_input_width, const int unpadded_output_width, const bool wait = true) {
         if (unpadded_input_width > int(get_input_width()) || unpadded_output_width > int(get_output_width()))
             throw std::invalid_argument("Padded weights width cannot be less than the unpadded.");
         constexpr int input_width_divisibly_by = 16;
@@ -169,14 +170,14 @@ template <typename T> class Network : public NetworkBase<T> {
             throw std::invalid_argument("one_padded_input_width > padded_input_width, the input width is too small.");
         const tnn_mlp_desc d = weights_desc();
         tnn::abi_check(tnn_zero_weights_padding(&d, m_weights_matrices.data(), unpadded_input_width, unpadded_output_width, use_bias_ ? 1 : 0, m_q.abi()));
-        m_q.wait();
+        if (wait) m_q.wait();
     }
 
-    void TransposeWeights(const DeviceMatrices<T> &weights, DeviceMatrices<T> &weightsT) {
+    void TransposeWeights(const DeviceMatrices<T> &weights, DeviceMatrices<T> &weightsT, const bool wait = true) {
         weights.PackedTranspose(weightsT);
         const tnn_mlp_desc d = weights_desc();
         tnn::abi_check(tnn_mlp_prepare_weights(&d, weights.data(), 0, prepared_fwd_, prepared_bwd_, m_q.abi()));
-        m_q.wait();
+        if (wait) m_q.wait();
     }
 
     void initialize_weights_matrices(const int unpadded_input_width, const int unpadded_output_width, WeightInitMode mode) {

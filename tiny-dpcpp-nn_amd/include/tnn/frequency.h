@@ -29,7 +29,6 @@ template <typename T> class FrequencyEncoding : public Encoding<T> {
         tnn::abi_check(tnn_frequency_forward(input.GetPointer(), this->get_input_width(), n_frequencies_, output->GetPointer(),
                                              tnn::dtype_of<T>::value, this->get_padded_output_width(), dy_dx, input.m(),
                                              this->get_queue().abi()));
-        this->get_queue().wait();
         return forward;
     }
 
@@ -46,7 +45,6 @@ template <typename T> class FrequencyEncoding : public Encoding<T> {
         tnn::abi_check(tnn_frequency_backward(dL_doutput.GetPointer(), tnn::dtype_of<T>::value, this->get_padded_output_width(),
                                               fwd.dy_dx.data(), this->get_input_width(), n_frequencies_, dL_dinput->data(), input.m(),
                                               this->get_queue().abi()));
-        this->get_queue().wait();
     }
 
   private:

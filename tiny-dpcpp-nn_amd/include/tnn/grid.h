@@ -82,8 +82,7 @@ template <typename T> class GridEncodingTemplated : public GridEncoding<T> {
         check_max_level();
         tnn::abi_check(tnn_grid_forward(&m_desc, input.GetPointer(), this->get_params()->data(), output->GetPointer(), TNN_FP32,
                                         this->get_padded_output_width(), input.m(), this->get_queue().abi()));
-        this->get_queue().wait();
-        return nullptr;
+        return nullptr; // enqueued on the encoding's in-order stream; the caller waits on the queue when it needs the host to see it
     }
 
     void backward_impl(const Context &, const DeviceMatrixView<float> input, const DeviceMatrixView<T> dL_doutput,

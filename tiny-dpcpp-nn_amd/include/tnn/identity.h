@@ -20,7 +20,6 @@ template <typename T> class IdentityEncoding : public Encoding<T> {
         if (input.stride() != input.n() || output->stride() != output->n()) throw std::invalid_argument("Only dense matrices are supported.");
         tnn::abi_check(tnn_identity_forward(input.GetPointer(), this->get_input_width(), m_scale, m_offset, output->GetPointer(),
                                             tnn::dtype_of<T>::value, this->get_padded_output_width(), input.m(), this->get_queue().abi()));
-        this->get_queue().wait();
         return std::make_unique<Context>();
     }
 

@@ -51,6 +51,13 @@ class Module {
 
     tnn::queue &get_queue() { return queue_; }
 
+    /// The reference blocks at the end of every method. Here the module's work and the tensor operations of the caller
+    /// share one in-order stream (torch's current stream, taken at construction), so the results are ordered without a
+    /// host wait; only when the caller has moved to another stream since does the method wait for the module's own.
+    void finish() {
+        if (c10::hip::getCurrentHIPStream().stream() != queue_.get()) queue_.wait();
+    }
+
     template <typename T> static std::vector<T> convertTensorToVector(const torch::Tensor &tensor) {
         const auto cpu = tensor.to(torch::kCPU).to(torch::kFloat32).contiguous();
         const float *begin = cpu.data_ptr<float>();
@@ -119,7 +126,7 @@ template <typename T> class EncodingModule : public Module {
         this->AllocateWorkspace(batch_size);
         DeviceMatrixView<T> output_encoding(batch_size, out_w, out_w, output_encoding_ptr_);
         std::unique_ptr<Context> model_ctx = encoding_->forward_impl(input_dmv, &output_encoding);
-        this->get_queue().wait();
+        this->finish();
         return fromDevice<T>(output_encoding.GetPointer(), {(int64_t)batch_size, (int64_t)out_w});
     }
 
@@ -155,7 +162,7 @@ template <typename T> class EncodingModule : public Module {
         auto gradients_view = gradients_->GetView();
         Context ctx;
         encoding_->backward_impl(ctx, input_encoding_dmv, dL_doutput_dmv, &gradients_view);
-        this->get_queue().wait();
+        this->finish();
         return {torch::Tensor(), convertDeviceMatrixToTorchTensor(*gradients_)};
     }
 
@@ -224,6 +231,8 @@ template <typename T, int WIDTH> class NetworkModule : public Module {
                    Network<T>::WeightInitMode::xavier_normal, use_bias),
           net_gradients_(network_.get_n_hidden_layers() + 1, network_.get_network_width(), WIDTH, WIDTH, WIDTH, WIDTH,
                          network_.get_output_width(), this->get_queue()),
+          net_gradients_packed_(network_.get_n_hidden_layers() + 1, network_.get_network_width(), WIDTH, WIDTH, WIDTH, WIDTH,
+                                network_.get_output_width(), this->get_queue()),
           max_batch_size_(0), interm_forw_ptr_(nullptr), interm_backw_ptr_(nullptr), dL_dinput_ptr_(nullptr) {
         net_gradients_.fill(T(0.0f)).wait();
     }
@@ -239,7 +248,7 @@ template <typename T, int WIDTH> class NetworkModule : public Module {
         this->AllocateWorkspace(batch_size);
         DeviceMatricesView<T> output_network(1, batch_size, network_.get_output_width(), 0, 0, 0, 0, interm_forw_ptr_);
         network_.inference(input_dm, output_network, {});
-        this->get_queue().wait();
+        this->finish();
         return fromDevice<T>(interm_forw_ptr_, {(int64_t)batch_size, out_w});
     }
 
@@ -252,7 +261,7 @@ template <typename T, int WIDTH> class NetworkModule : public Module {
         this->AllocateWorkspace(batch_size);
         DeviceMatricesView<T> output_network = ForwardViews(batch_size);
         network_.forward_pass(input_dm, output_network, {});
-        this->get_queue().wait();
+        this->finish();
         forward_batch_size_ = batch_size;
         return fromDevice<T>(output_network.GetMatrixPointer(network_.get_n_hidden_layers() + 1), {(int64_t)batch_size, out_w});
     }
@@ -284,14 +293,20 @@ template <typename T, int WIDTH> class NetworkModule : public Module {
         DeviceMatrixView<T> dL_dinput(batch_size, network_.get_input_width(), network_.get_input_width(), dL_dinput_ptr_);
 
         network_.backward_pass(dL_doutput, net_gradients_.GetViews(), interm_bwd, interm_fwd, {}, get_dl_dinput ? &dL_dinput : nullptr);
-        this->get_queue().wait();
+        this->finish();
 
-        // Pack and transpose: the kernels compute x * W, torch-style gradients are laid out for W * x
-        if (pack_transpose_gradient) net_gradients_.PackAndTranspose(net_gradients_);
+        // Pack and transpose: the kernels compute x * W, torch-style gradients are laid out for W * x. The reference does it in
+        // place (through a temporary); here the packed copy has a buffer of its own, so nothing is allocated per call.
+        const DeviceMatrices<T> *result = &net_gradients_;
+        if (pack_transpose_gradient) {
+            net_gradients_.PackAndTranspose(net_gradients_packed_);
+            this->finish();
+            result = &net_gradients_packed_;
+        }
 
         torch::Tensor input_grad;
         if (get_dl_dinput) input_grad = fromDevice<T>(dL_dinput.GetPointer(), {(int64_t)dL_dinput.nelements(), 1});
-        return {input_grad, fromDevice<T>(net_gradients_.GetViews().GetMatrixPointer(0), {(int64_t)net_gradients_.nelements(), 1})};
+        return {input_grad, fromDevice<T>(result->GetViews().GetMatrixPointer(0), {(int64_t)result->nelements(), 1})};
     }
 
     torch::Tensor initialize_params() override { return get_params(); }
@@ -329,7 +344,7 @@ template <typename T, int WIDTH> class NetworkModule : public Module {
     }
 
     std::vector<T> get_network_params() { return network_.get_weights_matrices().copy_to_host(); }
-    std::vector<T> get_network_grads() { return net_gradients_.copy_to_host(); }
+    std::vector<T> get_network_grads() { return net_gradients_.copy_to_host(); } // raw layout
 
   protected:
     void AllocateWorkspace(const size_t batch_size) override {
@@ -374,7 +389,8 @@ template <typename T, int WIDTH> class NetworkModule : public Module {
     }
 
     SwiftNetMLP<T, WIDTH> network_;
-    DeviceMatrices<T> net_gradients_; // independent of the batch size
+    DeviceMatrices<T> net_gradients_; // independent of the batch size; raw [out][in] as the backward pass writes them
+    DeviceMatrices<T> net_gradients_packed_; // the same in the parameter layout
     size_t max_batch_size_;           // the workspaces fit every batch size seen so far
     size_t forward_batch_size_ = 0;   // batch size of the activations held in interm_forw_ptr_
     T *interm_forw_ptr_;

@@ -259,6 +259,16 @@ int tnn_grid_forward(const tnn_grid_desc *desc, const float *d_x, const void *d_
 int tnn_grid_backward(const tnn_grid_desc *desc, const float *d_x, const void *d_dLdy, int dy_dtype,
                       uint32_t padded_width, float *d_grad_table, int overwrite, size_t M, tnn_stream_t stream);
 
+/* The same scatter into an fp16 gradient table, two features of an entry per packed atomic (global_atomic_pk_add_f16): half
+ * as many atomic operations as the fp32 route, which is what bounds the pass. No counterpart in the reference, whose
+ * gradients are float (grad_t, include/encodings/grid.h:586, "we don't have atomics for half precision",
+ * dpcpp_bindings/tiny_dpcpp_nn/modules.py:320-324); it is what tiny-cuda-nn does for half-precision grids. Sums are
+ * rounded to fp16 at every addition: scale dL/dy (loss scale) so that contributions stay clear of fp16's denormal range.
+ * n_features_per_level must be even. d_grad_table_f16: n_params fp16. Coarse levels are still accumulated in fp32 (LDS)
+ * and rounded once when they are flushed. */
+int tnn_grid_backward_packed(const tnn_grid_desc *desc, const float *d_x, const void *d_dLdy, int dy_dtype,
+                             uint32_t padded_width, void *d_grad_table_f16, int overwrite, size_t M, tnn_stream_t stream);
+
 /* Debug/verification aid: entry index (inside its level) of every (point, level, corner), the
  * integer part of kernel_grid (grid.h:95-129 with grid_index, common_device.h:745-765).
  * d_indices: M x n_levels x 2^n_dims uint32. */

@@ -182,3 +182,30 @@ def test_baseline_config_4_backward_full_size(tnn, oracle):
     # relative to the sum of magnitudes
     mag = float((out.double().abs() * g.double().abs()).sum())
     assert abs(lhs - rhs) <= 1e-6 * mag
+
+
+@pytest.mark.parametrize("cfg,M", [(CFG4, 1 << 16), (CFG5, 1 << 15), (dict(CFG4, n_features_per_level=4, n_levels=8), 5000)])
+def test_backward_packed_fp16_table(tnn, oracle, cfg, M):
+    """tnn_grid_backward_packed: same scatter, fp16 table, one packed atomic per pair of features. Every addition rounds to
+    fp16, so an entry that receives n contributions is within about sqrt(n) * 2^-11 of the fp32 sum: 2e-2 of the largest
+    entry per element, 2e-3 in the Frobenius norm. Overwrite zeroes the table first, Accumulate adds to it."""
+    from gpu_harness import ptr
+    from tiny_dpcpp_nn import _lib
+    d = tnn.grid_desc(cfg, FP16)
+    n = tnn.grid_n_params(d)
+    D = cfg["n_dims"]
+    pw = cfg["n_levels"] * cfg["n_features_per_level"]
+    gen = torch.Generator(device=tnn.dev).manual_seed(8)
+    x = torch.rand((M, D), device=tnn.dev, generator=gen)
+    g = (torch.rand((M, pw), device=tnn.dev, generator=gen) - 0.5).to(torch.float16)
+    table = torch.full((n,), 7.0, dtype=torch.float16, device=tnn.dev)
+    _lib.check(tnn.lib.tnn_grid_backward_packed(ctypes.byref(d), ptr(x), ptr(g), FP16, pw, ptr(table), 1, M, tnn.stream()))
+    ref = oracle.grid_backward(cfg, x.cpu().numpy(), g.float().cpu().numpy(), n)
+    got = table.float().cpu().numpy()
+    top = np.abs(ref).max()
+    assert np.abs(got - ref).max() <= 2e-2 * top
+    assert np.linalg.norm(got - ref) <= 2e-3 * np.linalg.norm(ref)
+    _lib.check(tnn.lib.tnn_grid_backward_packed(ctypes.byref(d), ptr(x), ptr(g), FP16, pw, ptr(table), 0, M, tnn.stream()))
+    assert np.linalg.norm(table.float().cpu().numpy() - 2 * ref) <= 4e-3 * np.linalg.norm(ref)
+    odd = tnn.grid_desc(dict(cfg, n_features_per_level=1), FP16)
+    assert tnn.lib.tnn_grid_backward_packed(ctypes.byref(odd), ptr(x), ptr(g), FP16, pw, ptr(table), 1, 8, tnn.stream()) == _lib.TNN_ERR_UNSUPPORTED

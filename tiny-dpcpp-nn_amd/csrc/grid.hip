@@ -295,6 +295,23 @@ __device__ __forceinline__ void for_each_corner(const float (&x)[D], float scale
     }
 }
 
+typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
+
+// Adds the F gradient values of one table entry. fp32 tables: one atomic per value (the reference's grad_t). fp16 tables:
+// one packed atomic (global_atomic_pk_add_f16) per pair of features, half as many atomic operations.
+template <int F> __device__ __forceinline__ void add_entry(float *entry, const float (&v)[F]) {
+#pragma unroll
+    for (int f = 0; f < F; ++f) unsafeAtomicAdd(entry + f, v[f]);
+}
+template <int F> __device__ __forceinline__ void add_entry(fp16_t *entry, const float (&v)[F]) {
+    static_assert(F % 2 == 0, "packed fp16 gradients need an even number of features per level");
+#pragma unroll
+    for (int f = 0; f < F; f += 2) {
+        const f16x2_t pair = {(fp16_t)v[f], (fp16_t)v[f + 1]};
+        (void)__builtin_amdgcn_flat_atomic_fadd_v2f16(reinterpret_cast<f16x2_t *>(entry + f), pair);
+    }
+}
+
 // Scatter-add of dL/dy into the gradient table (include/encodings/grid.h:137-245 of the reference: float atomics,
 // order not defined). Two routes inside one launch:
 //   * small levels (the coarse ones, where every point of the batch lands on a few hundred entries and global
@@ -302,10 +319,10 @@ __device__ __forceinline__ void for_each_corner(const float (&x)[D], float scale
 //     private copy of the level in LDS and then issues one global atomic per touched entry;
 //   * the other levels: one thread per (point, level), atomics straight to the table; workgroups of one level
 //     are dispatched together, so its slice of the table is the hot one in L2.
-template <int D, int F, typename G>
+template <int D, int F, typename G, typename GT>
 __global__ void __launch_bounds__(kGridThreads)
     grid_backward_kernel(const GridLevels lv, const GridParams gp, const BackwardPlan bp, const float *__restrict__ xin,
-                         const G *__restrict__ dLdy, float *__restrict__ grad, long long M) {
+                         const G *__restrict__ dLdy, GT *__restrict__ grad, long long M) {
     extern __shared__ float priv[];
     const uint32_t n_small_blocks = bp.n_small * bp.small_blocks;
     if (blockIdx.x < n_small_blocks) {
@@ -330,10 +347,16 @@ __global__ void __launch_bounds__(kGridThreads)
             });
         }
         __syncthreads();
-        float *g = grad + (size_t)lv.offset[l] * F;
-        for (uint32_t e = threadIdx.x; e < n; e += kGridThreads) {
-            const float v = priv[e];
-            if (v != 0.0f) unsafeAtomicAdd(g + e, v);
+        GT *g = grad + (size_t)lv.offset[l] * F;
+        for (uint32_t e = threadIdx.x; e < size; e += kGridThreads) {
+            float v[F];
+            bool any = false;
+#pragma unroll
+            for (int f = 0; f < F; ++f) {
+                v[f] = priv[e * F + f];
+                any |= v[f] != 0.0f;
+            }
+            if (any) add_entry<F>(g + (size_t)e * F, v);
         }
         return;
     }
@@ -347,11 +370,13 @@ __global__ void __launch_bounds__(kGridThreads)
     float gy[F];
 #pragma unroll
     for (int f = 0; f < F; ++f) gy[f] = (float)dLdy[i * gp.padded_width + l * F + f];
-    float *g = grad + (size_t)lv.offset[l] * F;
+    GT *g = grad + (size_t)lv.offset[l] * F;
     for_each_corner<D>(x, lv.scale[l], lv.size[l], lv.resolution[l], lv.flags[l], gp.hash_type, gp.interpolation,
                        [&](uint32_t idx, float w) {
+                           float v[F];
 #pragma unroll
-                           for (int f = 0; f < F; ++f) unsafeAtomicAdd(g + (size_t)idx * F + f, w * gy[f]);
+                           for (int f = 0; f < F; ++f) v[f] = w * gy[f];
+                           add_entry<F>(g + (size_t)idx * F, v);
                        });
 }
 
@@ -404,9 +429,9 @@ static int launch_grid_forward_p(const tnn_grid_desc *d, const GridLevels &lv, c
     return launch_grid_forward_o<D, F, fp16_t>(lv, gp, x, table, out, out_dtype, M, s);
 }
 
-template <int D, int F>
+template <int D, int F, typename TAB>
 static int launch_grid_backward_g(const GridLevels &lv, const GridParams &gp, const float *x, const void *dLdy, int dy_dtype,
-                                  float *grad, size_t M, hipStream_t s) {
+                                  TAB *grad, size_t M, hipStream_t s) {
     // A level goes the LDS route when its slice fits the budget and a chunk of points makes clearly more atomics
     // than the flush of the private copy does (chunk * 2^D contributions against `size` entries).
     BackwardPlan bp{};
@@ -429,7 +454,7 @@ static int launch_grid_backward_g(const GridLevels &lv, const GridParams &gp, co
     const dim3 grid((unsigned)blocks);
 #define TNN_BWD(GT)                                                                                                    \
     do {                                                                                                               \
-        auto k = grid_backward_kernel<D, F, GT>;                                                                       \
+        auto k = grid_backward_kernel<D, F, GT, TAB>;                                                                  \
         if (lds_bytes > 48 * 1024 &&                                                                                   \
             hipFuncSetAttribute(reinterpret_cast<const void *>(k), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes) != hipSuccess) \
             return fail(TNN_ERR_HIP, "cannot reserve %u bytes of LDS", lds_bytes);                                     \
@@ -554,28 +579,53 @@ TNN_API int tnn_grid_forward(const tnn_grid_desc *desc, const float *d_x, const 
     return rc;
 }
 
-TNN_API int tnn_grid_backward(const tnn_grid_desc *desc, const float *d_x, const void *d_dLdy, int dy_dtype,
-                              uint32_t padded_width, float *d_grad_table, int overwrite, size_t M, tnn_stream_t stream) {
+static int grid_backward_any(const tnn_grid_desc *desc, const float *d_x, const void *d_dLdy, int dy_dtype, uint32_t padded_width,
+                             void *d_grad_table, int grad_dtype, int overwrite, size_t M, tnn_stream_t stream) {
     GridLevels lv;
     GridParams gp;
     int rc = grid_common(desc, padded_width, M, &lv, &gp);
     if (rc) return rc;
     if (!d_x || !d_dLdy || !d_grad_table) return fail(TNN_ERR_INVALID_ARGUMENT, "NULL pointer argument");
+    if (grad_dtype != TNN_FP32 && grad_dtype != TNN_FP16) return fail(TNN_ERR_UNSUPPORTED, "gradient table dtype %d", grad_dtype);
+    if (grad_dtype == TNN_FP16 && desc->n_features_per_level % 2 != 0)
+        return fail(TNN_ERR_UNSUPPORTED, "fp16 gradient tables need an even number of features per level (features are added in pairs)");
     hipStream_t s = as_stream(stream);
     if (overwrite) {
         // a fill kernel rather than a memset node, so the call can be captured into a HIP graph
-        const size_t n = tnn_grid_n_params(desc);
+        const size_t bytes = tnn_grid_n_params(desc) * (grad_dtype == TNN_FP32 ? sizeof(float) : sizeof(fp16_t));
         if (reinterpret_cast<uintptr_t>(d_grad_table) & 15) return fail(TNN_ERR_INVALID_ARGUMENT, "d_grad_table must be 16-byte aligned");
-        const size_t n4 = n / 4;
-        const size_t n_tail = n - n4 * 4;
+        const size_t n4 = bytes / 16;
+        const size_t n_tail = (bytes - n4 * 16) / sizeof(float); // level sizes are multiples of 8 entries: fp16 tables leave no tail
         size_t blocks = (n4 + 255) / 256;
         if (blocks > 4096) blocks = 4096;
         if (blocks < 4) blocks = 4;
-        TNN_LAUNCH(fill_zero_kernel, dim3((unsigned)blocks), dim3(256), 0, s, (float4 *)d_grad_table, n4, d_grad_table + n4 * 4, n_tail);
+        TNN_LAUNCH(fill_zero_kernel, dim3((unsigned)blocks), dim3(256), 0, s, (float4 *)d_grad_table, n4,
+                   reinterpret_cast<float *>(static_cast<char *>(d_grad_table) + n4 * 16), n_tail);
         if ((rc = check_launch("fill_zero_kernel"))) return rc;
     }
-    TNN_DISPATCH_DF(desc, rc = (launch_grid_backward_g<D_, F_>(lv, gp, d_x, d_dLdy, dy_dtype, d_grad_table, M, s)));
+    if (grad_dtype == TNN_FP32) {
+        TNN_DISPATCH_DF(desc, rc = (launch_grid_backward_g<D_, F_, float>(lv, gp, d_x, d_dLdy, dy_dtype, (float *)d_grad_table, M, s)));
+    } else {
+        const uint32_t F = desc->n_features_per_level;
+#define TNN_PACKED(D_, F_) rc = launch_grid_backward_g<D_, F_, fp16_t>(lv, gp, d_x, d_dLdy, dy_dtype, (fp16_t *)d_grad_table, M, s)
+        if (desc->n_dims == 2) {
+            if (F == 2) TNN_PACKED(2, 2); else if (F == 4) TNN_PACKED(2, 4); else TNN_PACKED(2, 8);
+        } else {
+            if (F == 2) TNN_PACKED(3, 2); else if (F == 4) TNN_PACKED(3, 4); else TNN_PACKED(3, 8);
+        }
+#undef TNN_PACKED
+    }
     return rc;
+}
+
+TNN_API int tnn_grid_backward(const tnn_grid_desc *desc, const float *d_x, const void *d_dLdy, int dy_dtype,
+                              uint32_t padded_width, float *d_grad_table, int overwrite, size_t M, tnn_stream_t stream) {
+    return grid_backward_any(desc, d_x, d_dLdy, dy_dtype, padded_width, d_grad_table, TNN_FP32, overwrite, M, stream);
+}
+
+TNN_API int tnn_grid_backward_packed(const tnn_grid_desc *desc, const float *d_x, const void *d_dLdy, int dy_dtype,
+                                     uint32_t padded_width, void *d_grad_table_f16, int overwrite, size_t M, tnn_stream_t stream) {
+    return grid_backward_any(desc, d_x, d_dLdy, dy_dtype, padded_width, d_grad_table_f16, TNN_FP16, overwrite, M, stream);
 }
 
 TNN_API int tnn_grid_indices(const tnn_grid_desc *desc, const float *d_x, uint32_t *d_indices, size_t M, tnn_stream_t stream) {

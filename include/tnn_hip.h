@@ -274,6 +274,21 @@ int tnn_grid_backward_packed(const tnn_grid_desc *desc, const float *d_x, const 
  * d_indices: M x n_levels x 2^n_dims uint32. */
 int tnn_grid_indices(const tnn_grid_desc *desc, const float *d_x, uint32_t *d_indices, size_t M, tnn_stream_t stream);
 
+/* Grid encoding and network inference in one kernel: y = MLP(pad(grid(x))), the encoded rows stay in registers.
+ * Replaces the pair of calls behind NetworkWithInputEncoding in inference
+ * (dpcpp_bindings/tiny_dpcpp_nn/modules.py:357-421: Encoding.forward, then Network.forward on its padded output;
+ * include/encodings/grid.h:37-135 + include/network/kernel_esimd.h:565-640) and returns the values of
+ * tnn_grid_forward(out_dtype = mlp->dtype, padded_width = mlp->width) followed by tnn_mlp_inference, bit for bit.
+ * Needs n_levels * n_features_per_level <= mlp->width and weights that fit LDS beside 2.5 KiB of level constants (width 64: up to
+ * 19 matrices, width 128: up to 4); TNN_ERR_UNSUPPORTED otherwise, and the two calls do the work.
+ * d_x: M x n_dims fp32. d_table: n_params of grid->param_dtype. d_prepared_fwd: tnn_mlp_prepare_weights' forward
+ * buffer. d_y: M x width of mlp->dtype. M: positive multiple of 8. */
+int tnn_grid_mlp_inference(const tnn_grid_desc *grid, const tnn_mlp_desc *mlp, const float *d_x, const void *d_table,
+                           const void *d_prepared_fwd, void *d_y, size_t M, tnn_stream_t stream);
+/* TNN_OK when tnn_grid_mlp_inference runs this pair of shapes, otherwise the status (and tnn_last_error the reason) it
+ * would return: lets a caller choose between the fused call and the two calls once, when the modules are built. */
+int tnn_grid_mlp_supported(const tnn_grid_desc *grid, const tnn_mlp_desc *mlp);
+
 /* ------------------------------------------------------------------------------------------
  * Encodings without parameters. Rows are M x padded_width of out_dtype; the columns beyond the encoding's own
  * width are filled with ONES (the grid pads with zeros). Inputs are M x n_dims fp32, row-major.

@@ -139,6 +139,13 @@ class Harness:
         _lib.check(self.lib.tnn_grid_forward(ctypes.byref(d), ptr(x_t), ptr(table_t), ptr(out), out_dtype, padded_width, M, self.stream()))
         return out
 
+    def grid_mlp_inference(self, gd, desc, x_t, table_t, prep_fwd):
+        M = x_t.shape[0]
+        y = torch.full((M, desc.width), float("nan"), dtype=TORCH_DT[desc.dtype], device=self.dev)
+        _lib.check(self.lib.tnn_grid_mlp_inference(ctypes.byref(gd), ctypes.byref(desc), ptr(x_t), ptr(table_t), ptr(prep_fwd), ptr(y), M,
+                                                   self.stream()))
+        return y
+
     def grid_backward(self, d, x_t, dLdy_t, dy_dtype, grad_t=None, overwrite=True):
         M, pw = dLdy_t.shape
         if grad_t is None:

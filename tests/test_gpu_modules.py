@@ -351,6 +351,33 @@ def test_parameter_free_encodings_through_the_package(tcnn, oracle):
         ident.set_params(torch.zeros(3, device=DEVICE))
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("n_dims, grid, batch", [(2, "GRID_2D", 1001), (3, "GRID_3D", 4096)])
+def test_network_with_grid_encoding_fused_inference(tcnn, dtype, n_dims, grid, batch):
+    """Evaluation without autograd takes the single-kernel route (encoding + network); with autograd enabled the two
+    modules run in turn. Same bits either way, also for a batch that is padded to a multiple of 8."""
+    cfg = dict(GRID_2D) if grid == "GRID_2D" else {"otype": "HashGrid", "n_levels": 16, "n_features_per_level": 2, "log2_hashmap_size": 15,
+                                                   "base_resolution": 16, "per_level_scale": 1.447}
+    torch.manual_seed(3)
+    model = tcnn.NetworkWithInputEncoding(n_dims, 5, net_config(64, 3), cfg, dtype=dtype, use_bias=False)
+    with torch.no_grad():
+        model.encoding.params.copy_(torch.rand_like(model.encoding.params) * 2 - 1)  # the initial table is +-1e-4
+    model.eval()
+    assert model.network.tnn_module.can_fuse_encoding(model.encoding.tnn_module)
+    x = torch.rand((batch, n_dims), device=DEVICE)
+    two_calls = model(x).detach()  # autograd on: Encoding.forward, then Network.forward
+    with torch.no_grad():
+        fused = model(x)
+    assert fused.shape == two_calls.shape == (batch, 5) and fused.dtype == dtype
+    assert float(two_calls.float().abs().max()) > 1e-3
+    assert torch.equal(fused.view(torch.int16), two_calls.view(torch.int16))
+    # an encoding without a grid, or a network whose weights do not fit LDS beside it, keeps the two calls
+    sh = tcnn.NetworkWithInputEncoding(3, 3, net_config(64, 2), {"otype": "SphericalHarmonics", "degree": 4}, dtype=dtype)
+    assert not sh.network.tnn_module.can_fuse_encoding(sh.encoding.tnn_module)
+    with pytest.raises(Exception, match="two calls"):
+        sh.network.tnn_module.inference_with_encoding(sh.encoding.tnn_module, torch.rand((8, 3), device=DEVICE))
+
+
 def test_nerf_style_directional_network(tcnn):
     """test/python/test_nerf_settings.py:80-86 of the reference: spherical harmonics of degree 4 feeding a network."""
     model = tcnn.NetworkWithInputEncoding(3, 3, net_config(64, 2), {"otype": "SphericalHarmonics", "degree": 4}, dtype=torch.bfloat16)

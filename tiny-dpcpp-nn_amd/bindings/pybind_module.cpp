@@ -53,6 +53,12 @@ class PybindingModule {
         CHECK_INPUT(grad_output);
         return m_module->backward_pass(grad_output, input_from_fwd, pack_gradient, get_dl_dinput);
     }
+    /// Network modules: whether inference on `encoding`'s output can run as one kernel, and that inference.
+    bool can_fuse_encoding(const PybindingModule &encoding) const { return m_module->can_fuse_encoding(*encoding.m_module); }
+    torch::Tensor inference_with_encoding(const PybindingModule &encoding, torch::Tensor positions) {
+        CHECK_INPUT(positions);
+        return m_module->inference_with_encoding(*encoding.m_module, positions);
+    }
     torch::Tensor initial_params() { return m_module->initialize_params(); }
     torch::Tensor initial_params(torch::Tensor &tensor) { return m_module->initialize_params(tensor); }
     /// weights_are_packed: the tensor already is in the packed parameter layout, no packing is done
@@ -108,6 +114,8 @@ PYBIND11_MODULE(tiny_dpcpp_nn_pybind_module, m) {
     py::class_<PybindingModule>(m, "Module")
         .def("fwd", &PybindingModule::fwd)
         .def("inference", &PybindingModule::inference)
+        .def("can_fuse_encoding", &PybindingModule::can_fuse_encoding)
+        .def("inference_with_encoding", &PybindingModule::inference_with_encoding)
         .def("bwd_no_encoding_grad", &PybindingModule::bwd_no_encoding_grad)
         .def("bwd_with_encoding_grad", &PybindingModule::bwd_with_encoding_grad)
         .def("initial_params", py::overload_cast<>(&PybindingModule::initial_params))

@@ -10,29 +10,12 @@
 // written as contiguous 16-byte pieces. Per-level constants (scale, resolution, table offset, size,
 // how many dimensions enter the dense index, whether the level is hashed) are evaluated once on the
 // host and reach the kernel as scalar kernel arguments; no thread evaluates exp2.
-#include "tnn_internal.h"
+#include "grid_device.h"
 
 #include <cmath>
 #include <cstring>
 
 namespace tnn {
-
-struct GridLevels {
-    uint32_t offset[TNN_GRID_MAX_LEVELS];  // entries
-    uint32_t size[TNN_GRID_MAX_LEVELS];    // entries in the level ("hashmap_size")
-    float scale[TNN_GRID_MAX_LEVELS];
-    uint32_t resolution[TNN_GRID_MAX_LEVELS];
-    // bits 0-3: number of dimensions that enter the strided index; bit 4: level is hashed;
-    // bit 5: size is a power of two
-    uint32_t flags[TNN_GRID_MAX_LEVELS];
-};
-
-struct GridParams {
-    uint32_t n_levels;
-    uint32_t hash_type;
-    uint32_t interpolation;
-    uint32_t padded_width;
-};
 
 // include/common/common_device.h:745-765 evaluated for the loop bounds only: the stride sequence
 // depends on (resolution, size, n_dims) and not on the position.
@@ -54,76 +37,8 @@ static void fill_levels(const tnn_grid_desc *d, GridLevels *lv) {
     }
 }
 
-template <int D> __device__ __forceinline__ uint32_t hash_pos(const uint32_t (&p)[D], uint32_t hash_type) {
-    // include/common/common_device.h:713-729
-    constexpr uint32_t prime[7] = {1958374283u, 2654435761u, 805459861u, 3674653429u, 2097192037u, 1434869437u, 2165219737u};
-    constexpr uint32_t coherent[7] = {1u, 2654435761u, 805459861u, 3674653429u, 2097192037u, 1434869437u, 2165219737u};
-    constexpr uint32_t reversed[7] = {2165219737u, 1434869437u, 2097192037u, 3674653429u, 805459861u, 2654435761u, 1958374283u};
-    uint32_t r = 0;
-    if (hash_type == TNN_HASH_COHERENT_PRIME) {
-#pragma unroll
-        for (int i = 0; i < D; ++i) r ^= p[i] * coherent[i];
-    } else if (hash_type == TNN_HASH_PRIME) {
-#pragma unroll
-        for (int i = 0; i < D; ++i) r ^= p[i] * prime[i];
-    } else if (hash_type == TNN_HASH_REVERSED_PRIME) {
-#pragma unroll
-        for (int i = 0; i < D; ++i) r ^= p[i] * reversed[i];
-    }
-    return r; // Rng hashes to 0, as in common_device.h:738-740
-}
-
-template <int D>
-__device__ __forceinline__ uint32_t level_index(const uint32_t (&p)[D], uint32_t size, uint32_t res, uint32_t flags,
-                                                uint32_t hash_type) {
-    uint32_t index;
-    if (flags & 16u) {
-        index = hash_pos<D>(p, hash_type);
-    } else {
-        const uint32_t dims_used = flags & 15u;
-        uint32_t stride = 1;
-        index = 0;
-#pragma unroll
-        for (int dim = 0; dim < D; ++dim) {
-            if ((uint32_t)dim < dims_used) {
-                index += p[dim] * stride;
-                stride *= res;
-            }
-        }
-    }
-    if (flags & 32u) return index & (size - 1);
-    return (index >= size) ? index % size : index;
-}
-
-// include/encodings/grid.h:73-93
-template <int D>
-__device__ __forceinline__ void cell_of(const float (&x)[D], float scale, uint32_t interpolation, uint32_t (&cell)[D],
-                                        float (&frac)[D]) {
-#pragma unroll
-    for (int d = 0; d < D; ++d) {
-        float p = __builtin_fmaf(scale, x[d], 0.5f);
-        const float t = floorf(p);
-        cell[d] = (uint32_t)(int)t;
-        p -= t;
-        frac[d] = (interpolation == TNN_INTERP_SMOOTHSTEP) ? p * p * (3.0f - 2.0f * p) : p;
-    }
-}
-
-template <typename P, int F> __device__ __forceinline__ void load_entry(const P *__restrict__ p, float (&v)[F]) {
-    // F consecutive features of one entry, fetched as a single vector load
-    typedef P vecF __attribute__((ext_vector_type(F)));
-    if (F == 1) {
-        v[0] = (float)p[0];
-    } else {
-        const vecF t = *reinterpret_cast<const vecF *>(p);
-#pragma unroll
-        for (int f = 0; f < F; ++f) v[f] = (float)t[f];
-    }
-}
-
-template <typename O> __device__ __forceinline__ O to_out(float v) { return (O)v; }
-
 constexpr int kGridThreads = 256;
+
 
 // Levels are processed in groups whose outputs fill one 16-byte piece of the encoded row: all gathers of a
 // group (GL * 2^D independent loads) are issued before the first blend, and the row is written in whole
@@ -145,67 +60,15 @@ __global__ void __launch_bounds__(kGridThreads)
     const bool row_aligned = ((gp.padded_width * sizeof(O)) % 16 == 0) && ((reinterpret_cast<uintptr_t>(out) & 15) == 0);
 
     for (uint32_t l0 = 0; l0 < gp.n_levels; l0 += GL) {
-        float vals[GL][1 << D][F];
-        float wts[GL][1 << D];
-        // gathers of the whole group
+        LevelConst lc[GL];
 #pragma unroll
-        for (int gl = 0; gl < GL; ++gl) {
-            const uint32_t l = l0 + gl;
-            if (l < gp.n_levels) {
-                const uint32_t size = lv.size[l], res = lv.resolution[l], flags = lv.flags[l];
-                const P *g = table + (size_t)lv.offset[l] * F;
-                uint32_t cell[D];
-                float frac[D];
-                cell_of<D>(x, lv.scale[l], gp.interpolation, cell, frac);
-                if (gp.interpolation == TNN_INTERP_NEAREST) {
-                    const uint32_t idx = level_index<D>(cell, size, res, flags, gp.hash_type);
-                    load_entry<P, F>(g + (size_t)idx * F, vals[gl][0]);
-                    wts[gl][0] = 1.0f;
-#pragma unroll
-                    for (int c = 1; c < (1 << D); ++c) {
-                        wts[gl][c] = 0.0f;
-#pragma unroll
-                        for (int f = 0; f < F; ++f) vals[gl][c][f] = 0.0f;
-                    }
-                } else {
-#pragma unroll
-                    for (int c = 0; c < (1 << D); ++c) {
-                        float weight = 1.0f;
-                        uint32_t loc[D];
-#pragma unroll
-                        for (int d = 0; d < D; ++d) {
-                            if ((c & (1 << d)) == 0) {
-                                weight *= 1 - frac[d];
-                                loc[d] = cell[d];
-                            } else {
-                                weight *= frac[d];
-                                loc[d] = cell[d] + 1;
-                            }
-                        }
-                        wts[gl][c] = weight;
-                        const uint32_t idx = level_index<D>(loc, size, res, flags, gp.hash_type);
-                        load_entry<P, F>(g + (size_t)idx * F, vals[gl][c]);
-                    }
-                }
-            }
-        }
-        // blends, in the corner order and with the fused multiply-add of include/encodings/grid.h:114-129
-        // (nearest: the single value is copied, grid.h:104-109)
+        for (int gl = 0; gl < GL; ++gl) lc[gl] = level_const(lv, (l0 + gl < gp.n_levels) ? l0 + gl : l0);
+        const int n_valid = (int)((gp.n_levels - l0 < (uint32_t)GL) ? gp.n_levels - l0 : (uint32_t)GL);
+        float r[NOUT];
+        encode_levels<D, F, P, GL>(lc, n_valid, gp, x, table, r);
         ovec o;
 #pragma unroll
-        for (int gl = 0; gl < GL; ++gl) {
-#pragma unroll
-            for (int f = 0; f < F; ++f) {
-                float r = 0.0f;
-                if (gp.interpolation == TNN_INTERP_NEAREST) {
-                    r = vals[gl][0][f];
-                } else {
-#pragma unroll
-                    for (int c = 0; c < (1 << D); ++c) r = __builtin_fmaf(wts[gl][c], vals[gl][c][f], r);
-                }
-                o[gl * F + f] = to_out<O>(r);
-            }
-        }
+        for (int e = 0; e < NOUT; ++e) o[e] = to_out<O>(r[e]);
         const uint32_t col0 = l0 * F;
         if (row_aligned && l0 + GL <= gp.n_levels) {
             if constexpr (NOUT * sizeof(O) == 16) {
@@ -387,7 +250,7 @@ __global__ void fill_zero_kernel(float4 *__restrict__ p, size_t n4, float *__res
     if (i < n_tail) tail[i] = 0.0f;
 }
 
-static int check_grid_desc(const tnn_grid_desc *d) {
+int check_grid_desc(const tnn_grid_desc *d) {
     if (!d) return fail(TNN_ERR_INVALID_ARGUMENT, "desc is NULL");
     if (d->n_dims != 2 && d->n_dims != 3) return fail(TNN_ERR_UNSUPPORTED, "GridEncoding: n_dims_to_encode %u (2 or 3 are built)", d->n_dims);
     if (d->n_levels == 0 || d->n_levels > TNN_GRID_MAX_LEVELS)
@@ -550,7 +413,8 @@ TNN_API size_t tnn_grid_n_params(const tnn_grid_desc *desc) {
     return (size_t)desc->offsets[desc->n_levels] * desc->n_features_per_level;
 }
 
-static int grid_common(const tnn_grid_desc *desc, uint32_t padded_width, size_t M, GridLevels *lv, GridParams *gp) {
+namespace tnn {
+int grid_common(const tnn_grid_desc *desc, uint32_t padded_width, size_t M, GridLevels *lv, GridParams *gp) {
     int rc = check_grid_desc(desc);
     if (rc) return rc;
     // include/encodings/grid.h:665-677
@@ -567,6 +431,7 @@ static int grid_common(const tnn_grid_desc *desc, uint32_t padded_width, size_t 
     gp->padded_width = padded_width;
     return TNN_OK;
 }
+} // namespace tnn
 
 TNN_API int tnn_grid_forward(const tnn_grid_desc *desc, const float *d_x, const void *d_table, void *d_out, int out_dtype,
                              uint32_t padded_width, size_t M, tnn_stream_t stream) {

@@ -52,6 +52,24 @@ template <typename T, int WIDTH> class SwiftNetMLP : public Network<T> {
         return {tnn::event(this->get_queue().get())};
     }
 
+    /// Whether inference_with_grid runs for this grid (its features fit the input width, the weights fit LDS).
+    bool supports_grid_input(const tnn_grid_desc &grid) const {
+        const tnn_mlp_desc d = desc();
+        return Network<T>::get_input_width() == WIDTH && tnn_grid_mlp_supported(&grid, &d) == TNN_OK;
+    }
+
+    /// Inference on the grid encoding of `positions` (M x n_dims fp32) without the encoded matrix ever being stored:
+    /// the same values as the encoding's forward_impl into a WIDTH-wide matrix of T followed by inference().
+    /// No counterpart in the reference, which runs the two kernels (dpcpp_bindings/tiny_dpcpp_nn/modules.py:357-421).
+    std::vector<tnn::event> inference_with_grid(const tnn_grid_desc &grid, const void *table, const float *positions, const size_t M,
+                                                DeviceMatricesView<T> output) {
+        if (Network<T>::get_input_width() != WIDTH) throw std::invalid_argument("The encoding must be padded to the network width.");
+        const tnn_mlp_desc d = desc();
+        tnn::abi_check(tnn_grid_mlp_inference(&grid, &d, positions, table, this->prepared_forward(), output.GetMatrixPointer(0), M,
+                                              this->get_queue().abi()));
+        return {tnn::event(this->get_queue().get())};
+    }
+
     /// input: dL/d(output). output: weight gradients, per matrix [out][in] row-major, unpacked.
     std::vector<tnn::event> backward_pass(const DeviceMatrix<T> &input, DeviceMatrices<T> &output,
                                           DeviceMatrices<T> &intermediate_output_backward,

@@ -49,6 +49,17 @@ class Module {
     virtual size_t n_params() = 0;
     virtual size_t n_output_dims() = 0;
 
+    /// Encoding modules whose encoding is a grid: its descriptor and its table on the device (nullptr otherwise).
+    virtual const tnn_grid_desc *grid_descriptor() const { return nullptr; }
+    virtual const void *grid_table() const { return nullptr; }
+    /// Network modules: inference on `encoding`'s output for `positions`, in one kernel, when can_fuse_encoding says so.
+    /// No counterpart in the reference (NetworkWithInputEncoding runs the two modules in turn,
+    /// dpcpp_bindings/tiny_dpcpp_nn/modules.py:357-421); the values are those of the two calls.
+    virtual bool can_fuse_encoding(const Module &) const { return false; }
+    virtual torch::Tensor inference_with_encoding(const Module &, const torch::Tensor &) {
+        throw std::runtime_error("inference_with_encoding: not a network module");
+    }
+
     tnn::queue &get_queue() { return queue_; }
 
     /// The reference blocks at the end of every method. Here the module's work and the tensor operations of the caller
@@ -189,6 +200,11 @@ template <typename T> class EncodingModule : public Module {
 
     size_t n_params() override { return encoding_->get_n_params(); }
     size_t n_output_dims() override { return encoding_->get_padded_output_width(); }
+    const tnn_grid_desc *grid_descriptor() const override {
+        const auto *grid = dynamic_cast<const tinydpcppnn::encodings::grid::GridEncodingTemplated<T> *>(encoding_.get());
+        return grid ? &grid->descriptor() : nullptr;
+    }
+    const void *grid_table() const override { return grid_descriptor() ? encoding_->get_params()->data() : nullptr; }
     std::vector<T> get_encoding_params() { return encoding_->get_params()->copy_to_host(); }
     std::vector<T> get_encoding_grads() { return gradients_->copy_to_host(); }
 
@@ -248,6 +264,30 @@ template <typename T, int WIDTH> class NetworkModule : public Module {
         this->AllocateWorkspace(batch_size);
         DeviceMatricesView<T> output_network(1, batch_size, network_.get_output_width(), 0, 0, 0, 0, interm_forw_ptr_);
         network_.inference(input_dm, output_network, {});
+        this->finish();
+        return fromDevice<T>(interm_forw_ptr_, {(int64_t)batch_size, out_w});
+    }
+
+    bool can_fuse_encoding(const Module &encoding) const override {
+        const tnn_grid_desc *grid = encoding.grid_descriptor();
+        return grid && network_.supports_grid_input(*grid);
+    }
+
+    torch::Tensor inference_with_encoding(const Module &encoding, const torch::Tensor &positions) override {
+        const tnn_grid_desc *grid = encoding.grid_descriptor();
+        if (!grid || !network_.supports_grid_input(*grid))
+            throw std::invalid_argument("inference_with_encoding: this encoding / network pair runs as two calls (" +
+                                        std::string(tnn_last_error()) + ")");
+        CHECK_INPUT(positions);
+        TORCH_CHECK(positions.dim() == 2 && positions.scalar_type() == torch::kFloat32, "positions must be a float32 matrix");
+        if (positions.sizes()[1] != (int64_t)grid->n_dims) throw std::runtime_error("Input tensor has incorrect dimensions");
+        if (positions.sizes()[0] % 8 != 0) throw std::invalid_argument("Batch size is not divisible by 8.");
+        const size_t batch_size = positions.sizes()[0];
+        const int64_t out_w = network_.get_output_width();
+        if (batch_size == 0) return torch::empty({0, out_w}, torch::TensorOptions().dtype(torch_type<T>::dtype).device(device()));
+        this->AllocateWorkspace(batch_size);
+        DeviceMatricesView<T> output_network(1, batch_size, network_.get_output_width(), 0, 0, 0, 0, interm_forw_ptr_);
+        network_.inference_with_grid(*grid, encoding.grid_table(), positions.data_ptr<float>(), batch_size, output_network);
         this->finish();
         return fromDevice<T>(interm_forw_ptr_, {(int64_t)batch_size, out_w});
     }

@@ -322,4 +322,18 @@ class NetworkWithInputEncoding(Module):
         self.network.set_params(params)
 
     def forward(self, x):
+        if (not self.training and not torch.is_grad_enabled() and x.shape[0] > 0
+                and self.network.tnn_module.can_fuse_encoding(self.encoding.tnn_module)):
+            return self._fused_inference(x)
         return self.network_with_encoding(x)
+
+    def _fused_inference(self, x):
+        """Evaluation without autograd on a grid encoding: encoding and network run as one kernel, the encoded matrix is
+        never stored. Same values as the two modules in turn (the reference's only route, modules.py:357-421)."""
+        batch_size = x.shape[0]
+        padded_batch_size = (batch_size + MIN_BATCH_SIZE - 1) // MIN_BATCH_SIZE * MIN_BATCH_SIZE
+        padded = x if batch_size == padded_batch_size else torch.nn.functional.pad(x, [0, 0, 0, padded_batch_size - batch_size])
+        self.encoding.set_params()
+        self.network.set_params()
+        output = self.network.tnn_module.inference_with_encoding(self.encoding.tnn_module, padded.to(torch.float32).contiguous())
+        return output.reshape(padded_batch_size, -1)[:batch_size, : self.n_output_dims]

@@ -27,12 +27,13 @@ PEAK_HBM = 8000.0  # GB/s
 
 # HBM-side bytes per launch of each workload's dominant kernel at the default batch sizes, from rocprofv3 counter runs over this
 # file (FETCH_SIZE and WRITE_SIZE, one run each, scaled by what the same counter reads for the --copy-calibration kernel:
-# x2.000 and x1.000). The summaries with the commands are profiles/mlp_train_fused_kernel.*.txt, profiles/mlp_forward_kernel.*.txt
-# and profiles/grid_forward_kernel.*.txt. Not measured live: counters need the profiler.
+# x2.000 and x1.000). The summaries with the commands are profiles/mlp_train_fused_kernel.*.txt, profiles/mlp_forward_kernel.*.txt,
+# profiles/grid_forward_kernel.*.txt and profiles/grid_mlp_inference_kernel.*.txt. Not measured live: counters need the profiler.
 MEASURED_TRAFFIC_BYTES = {
-    ("train", 18): (57794.4 * 2.0 + 20488.0) * 1024,
-    ("infer", 18): (16573.3 * 2.0 + 32768.0) * 1024,
-    ("grid", 21): (6156642.8 * 2.0 + 262143.8) * 1024,
+    ("train", 18): (57794.2 * 2.0 + 20488.0) * 1024,
+    ("infer", 18): (16573.3 * 2.0 + 32768.7) * 1024,
+    ("grid", 21): (6226188.0 * 2.0 + 262133.8) * 1024,
+    ("grid_mlp", 21): (6641648.3 * 2.0 + 263928.2) * 1024,
 }
 
 
@@ -41,7 +42,7 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="train", choices=["train", "infer", "grid"])
+    ap.add_argument("--workload", default="train", choices=["train", "infer", "grid", "grid_mlp"])
     ap.add_argument("--batch-log2", type=int, default=None)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -118,6 +119,33 @@ def cpu_baseline_grid(oracle, cfg, budget_s=12.0):
     dt = time.perf_counter() - t0
     return {"value": M * k / dt, "unit": "points/s", "cores": oracle.num_threads(), "kind": "port",
             "sample": f"{k} forward passes of {M} points through the full 162 MiB table, OpenMP over points"}
+
+
+def cpu_baseline_grid_mlp(oracle, cfg, w, budget_s=12.0):
+    import numpy as np
+    from tolerances import FP16
+
+    rng = np.random.default_rng(0)
+    off, _, _ = oracle.grid_offsets(cfg["n_dims"], cfg["n_levels"], cfg["log2_hashmap_size"], cfg["base_resolution"], cfg["per_level_scale"])
+    n = int(off[-1]) * cfg["n_features_per_level"]
+    table = oracle.round(rng.uniform(-1e-4, 1e-4, n), FP16)
+    M = 1 << 16
+    x = rng.uniform(0, 1, (M, cfg["n_dims"])).astype(np.float32)
+    n_mats = w.shape[0]
+
+    def chain():
+        enc = oracle.round(oracle.grid_forward(cfg, table, x, 64), FP16)
+        return oracle.mlp_forward_T(FP16, 64, n_mats, "relu", "none", w, enc, store_interm=False)
+
+    chain()
+    t0 = time.perf_counter()
+    k = 0
+    while time.perf_counter() - t0 < budget_s:
+        chain()
+        k += 1
+    dt = time.perf_counter() - t0
+    return {"value": M * k / dt, "unit": "points/s", "cores": oracle.num_threads(), "kind": "port",
+            "sample": f"{k} passes of {M} points: encoding through the full 162 MiB table, then the 4-matrix network, OpenMP over points"}
 
 
 def main():
@@ -274,32 +302,53 @@ def main():
         gen = torch.Generator(device=t.dev).manual_seed(7)
         table = (torch.rand(n, device=t.dev, generator=gen) * 2e-4 - 1e-4).to(torch.float16)
         x = torch.rand((M, 3), device=t.dev, generator=gen)
-        o = torch.empty((M, 32), dtype=torch.float16, device=t.dev)
         s = t.stream()
         K = min(K, 50)
+        if args.workload == "grid":
+            o = torch.empty((M, 32), dtype=torch.float16, device=t.dev)
+            call = lambda: lib.tnn_grid_forward(ctypes.byref(gd), ptr(x), ptr(table), ptr(o), FP16, 32, M, s)
+            bpp = 12 + 16 * 8 * 4 + 32 * 2
+        else:
+            # BASELINE config 5 whole: the encoding feeds a width-64 network with 3 hidden layers (16 real outputs) in one kernel
+            W, n_hidden, n_out = 64, 3, 16
+            mdesc = t.mlp_desc(FP16, W, n_hidden, "relu", "none")
+            rng = np.random.default_rng(42)
+            lim = np.sqrt(6.0 / (2 * W))
+            w = rng.uniform(-lim, lim, (n_hidden + 1, W, W)).astype(np.float32)
+            w[0, 32:, :] = 0
+            w[-1, :, n_out:] = 0
+            _, pf, _ = t.prepare(mdesc, w)
+            o = torch.empty((M, W), dtype=torch.float16, device=t.dev)
+            call = lambda: lib.tnn_grid_mlp_inference(ctypes.byref(gd), ctypes.byref(mdesc), ptr(x), ptr(table), ptr(pf), ptr(o), M, s)
+            bpp = 12 + 16 * 8 * 4 + W * 2  # coordinates + gathers + the padded output row; the encoded row stays on chip
         for _ in range(min(Wm, 5)):
-            lib.tnn_grid_forward(ctypes.byref(gd), ptr(x), ptr(table), ptr(o), FP16, 32, M, s)
+            rc = call()
+            if rc:
+                raise RuntimeError(lib.tnn_last_error())
         torch.cuda.synchronize()
         e0, e1 = ev(), ev()
         e0.record()
         for _ in range(K):
-            lib.tnn_grid_forward(ctypes.byref(gd), ptr(x), ptr(table), ptr(o), FP16, 32, M, s)
+            call()
         e1.record()
         torch.cuda.synchronize()
         ms = e0.elapsed_time(e1) / K
-        bpp = 12 + 16 * 8 * 4 + 32 * 2
+        grid_only = args.workload == "grid"
         out = {
-            "metric": "hash-grid forward points/s (3-D, 16x2, log2 22, fp16 table, batch 2^21); % HBM peak",
+            "metric": ("hash-grid forward points/s (3-D, 16x2, log2 22, fp16 table, batch 2^21); % HBM peak" if grid_only else
+                       "hash-grid + fused-MLP inference points/s (3-D, 16x2, log2 22, fp16; w64, 3 hidden layers; batch 2^21); % HBM peak"),
             "value": M / (ms * 1e-3), "unit": "points/s", "n_gpus": 1, "steps": K, "warmup": min(Wm, 5), "ms_per_step": ms,
             "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
-            "config": {"workload": f"3-D hash-grid encoding forward, 2^{int(np.log2(M))} points (BASELINE config 5 encoding)", "batch": M},
+            "config": {"workload": (f"3-D hash-grid encoding forward, 2^{int(np.log2(M))} points (BASELINE config 5 encoding)" if grid_only else
+                                    f"3-D hash-grid encoding + w64/3-hidden-layer network inference in one kernel, 2^{int(np.log2(M))} points "
+                                    "(BASELINE config 5)"), "batch": M},
             "roofline": {"bound": "hbm", "achieved": bpp * M / (ms * 1e-3) / 1e9, "peak": PEAK_HBM, "unit": "GB/s",
-                         "frac": bpp * M / (ms * 1e-3) / 1e9 / PEAK_HBM, "traffic": MEASURED_TRAFFIC_BYTES.get(("grid", int(np.log2(M)))),
-                         "kernel": "grid_forward_kernel",
+                         "frac": bpp * M / (ms * 1e-3) / 1e9 / PEAK_HBM, "traffic": MEASURED_TRAFFIC_BYTES.get((args.workload, int(np.log2(M)))),
+                         "kernel": "grid_forward_kernel" if grid_only else "grid_mlp_inference_kernel",
                          "kernel_ms": ms, "algorithmic_bytes_per_launch": bpp * M},
         }
         if oracle is not None:
-            out["cpu_baseline"] = cpu_baseline_grid(oracle, cfg)
+            out["cpu_baseline"] = cpu_baseline_grid(oracle, cfg) if grid_only else cpu_baseline_grid_mlp(oracle, cfg, oracle.round(w, FP16))
 
     if args.copy_calibration:
         n = 64 << 20

@@ -369,3 +369,29 @@ def test_baseline_config_3_full_size(tnn, oracle, W, n_hidden):
     diff, bar = np.abs(dXh - rdX), 5e-4 * np.abs(rdX).max() + 5e-3 * np.abs(rdX)
     assert (diff <= bar).all(axis=1).mean() >= 0.98
     assert np.linalg.norm((dXh - rdX).ravel()) <= 2e-2 * np.linalg.norm(rdX.ravel())
+
+
+@pytest.mark.parametrize("dtype,W,n_hidden,log2_m", [(FP16, 16, 2, 19), (FP16, 16, 4, 19), (BF16, 32, 2, 19), (BF16, 64, 4, 18), (FP16, 64, 2, 17)])
+def test_train_step_is_reproducible(tnn, oracle, dtype, W, n_hidden, log2_m):
+    """The same step on the same data gives the same bits, every time: the partial sums are added in a fixed order and
+    nothing in the kernel depends on timing. Batches of several rounds per wave; width 16 is the shape in which half of
+    every weight-gradient accumulator is unused, which is where a register written behind the compiler's back (inline asm
+    next to an MFMA in flight) once made the result vary from run to run."""
+    import torch
+    M, n_mats = 1 << log2_m, n_hidden + 1
+    w = oracle.round(xavier(W, n_mats, 5), dtype)
+    desc = tnn.mlp_desc(dtype, W, n_hidden, "relu", "none")
+    _, pf, pb = tnn.prepare(desc, w)
+    gen = torch.Generator(device=tnn.dev).manual_seed(9)
+    x = (torch.rand((M, W), device=tnn.dev, generator=gen) * 2 - 1).to(torch.float16 if dtype == FP16 else torch.bfloat16)
+    targets = torch.rand((M, W), device=tnn.dev, generator=gen)
+    first = None
+    for _ in range(4):
+        y, loss, dW, dX = tnn.train_step_l2(desc, pf, pb, x, targets, 128.0 * M / 1024, want_dx=True, dw_fp32=True)
+        tnn.sync()
+        got = (y.clone(), loss.clone(), dW.clone(), dX.clone())
+        if first is None:
+            first = got
+        else:
+            for a, b in zip(got, first):
+                assert torch.equal(a.view(torch.int16 if a.element_size() == 2 else torch.int32), b.view(torch.int16 if b.element_size() == 2 else torch.int32))

@@ -44,26 +44,32 @@ __device__ __forceinline__ unsigned int relu_pair(unsigned int v) {
     return __builtin_bit_cast(unsigned int, b);
 }
 
+// Hides from the optimiser what a value is (here: that a mask is 0 or 1 per half, which it would turn back into
+// per-half compares and selects). The statement emits no instruction: the value stays in the register the compiler
+// gave it. Instructions written out in inline asm are not an option in these kernels: their destination registers are
+// invisible to the compiler's hazard bookkeeping, and one that lands in the unused part of the destination of an MFMA
+// still in flight is overwritten when the MFMA retires.
+__device__ __forceinline__ unsigned int opaque(unsigned int v) {
+    asm("" : "+v"(v));
+    return v;
+}
+
 // g where fwd > 0, else 0, with packed 16-bit integer instructions: m = min(max(fwd, 0), 1) is 1 exactly
-// for the positive values of fwd (as int16), and g * m keeps or clears the bit pattern of g. Written as
-// instructions because the compiler turns the 0/1 multiply back into per-half compares and selects.
+// for the positive values of fwd (as int16), and g * m keeps or clears the bit pattern of g
+// (v_pk_max_i16, v_pk_min_i16, v_pk_mul_lo_u16).
 __device__ __forceinline__ unsigned int relu_gate_pair(unsigned int g, unsigned int fwd) {
-    unsigned int m, r;
-    const unsigned int zero = 0u, one = 0x00010001u;
-    asm("v_pk_max_i16 %0, %1, %2" : "=v"(m) : "v"(fwd), "v"(zero));
-    asm("v_pk_min_i16 %0, %1, %2" : "=v"(m) : "v"(m), "v"(one));
-    asm("v_pk_mul_lo_u16 %0, %1, %2" : "=v"(r) : "v"(g), "v"(m));
-    return r;
+    s16x2 m = __builtin_elementwise_max(__builtin_bit_cast(s16x2, fwd), s16x2{0, 0});
+    m = __builtin_elementwise_min(m, __builtin_bit_cast(s16x2, opaque(0x00010001u)));
+    const u16x2 r = __builtin_bit_cast(u16x2, g) * __builtin_bit_cast(u16x2, opaque(__builtin_bit_cast(unsigned int, m)));
+    return __builtin_bit_cast(unsigned int, r);
 }
 
 // The same gate when fwd is known to be the output of relu_pair (never negative, never -0): min(fwd, 1)
-// as unsigned 16-bit integers is already the 0/1 mask.
+// as unsigned 16-bit integers is already the 0/1 mask (v_pk_min_u16, v_pk_mul_lo_u16).
 __device__ __forceinline__ unsigned int relu_gate_pair_nonneg(unsigned int g, unsigned int fwd) {
-    unsigned int m, r;
-    const unsigned int one = 0x00010001u;
-    asm("v_pk_min_u16 %0, %1, %2" : "=v"(m) : "v"(fwd), "v"(one));
-    asm("v_pk_mul_lo_u16 %0, %1, %2" : "=v"(r) : "v"(g), "v"(m));
-    return r;
+    const u16x2 m = __builtin_elementwise_min(__builtin_bit_cast(u16x2, fwd), __builtin_bit_cast(u16x2, opaque(0x00010001u)));
+    const u16x2 r = __builtin_bit_cast(u16x2, g) * __builtin_bit_cast(u16x2, opaque(__builtin_bit_cast(unsigned int, m)));
+    return __builtin_bit_cast(unsigned int, r);
 }
 
 // Accumulator half (8 fp32 of one 32x32 tile) -> activation -> 8 values of T.

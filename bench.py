@@ -151,8 +151,9 @@ def cpu_baseline_grid_mlp(oracle, cfg, w, budget_s=12.0):
 def main():
     args = parse()
     if args.gpus != 1:
-        print("bench.py measures one GPU: this build has no multi-GPU path (every row is independent; see DESIGN.md "
-              "for how it would shard). Run with --gpus 1.", file=sys.stderr)
+        print("bench.py measures one GPU: this build has no multi-GPU path. Every batch row is independent, so G GPUs would each take "
+              "M/G rows with a full copy of the weights and exchange the weight gradients once per step; that is not built. "
+              "Run with --gpus 1.", file=sys.stderr)
         sys.exit(2)
 
     import numpy as np

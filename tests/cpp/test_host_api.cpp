@@ -174,6 +174,41 @@ static void test_json() {
     CHECK(json::parse(j.dump())["n_levels"].get<int>() == 16);
 }
 
+// File helpers of io.h: what one writes the other reads back; formats as the reference's own files use them
+// (one value per line for weights, delimiter-separated rows for target vectors, binary PGM for images).
+static void test_io_files() {
+    const std::string dir = "/tmp/tnn_io_test_";
+    const std::vector<float> values{0.5f, -1.25f, 3.0f, 1e-3f};
+    io::saveCSV(dir + "v.csv", values);
+    CHECK(io::loadCSV(dir + "v.csv") == values);
+    CHECK(io::loadVectorFromCSV<float>(dir + "v.csv") == values);
+    CHECK(io::loadCSV(dir + "missing.csv").empty());
+    CHECK(throws<std::invalid_argument>([&] { io::loadVectorFromCSV<float>(dir + "missing.csv"); }));
+    {
+        std::ofstream f(dir + "t.csv");
+        f << "1;2;3\n4.5;-6\n";
+    }
+    const auto rows = io::readTargetVectorsFromFile(dir + "t.csv", ';');
+    CHECK(rows.size() == 2 && rows[0] == (std::vector<float>{1.f, 2.f, 3.f}) && rows[1] == (std::vector<float>{4.5f, -6.f}));
+    CHECK(io::readTargetVectorsFromFile(dir + "missing.csv", ',').empty());
+    const std::vector<unsigned char> image{0, 64, 128, 255, 1, 2};
+    io::saveImageToPGM(dir + "i.pgm", 3, 2, image);
+    std::ifstream f(dir + "i.pgm", std::ios::binary);
+    std::string bytes((std::istreambuf_iterator<char>(f)), std::istreambuf_iterator<char>());
+    CHECK(bytes == std::string("P5\n3 2\n255\n") + std::string(image.begin(), image.end()));
+    // unpacked [in][out] matrices, one value per line -> the packed parameter vector of a width-16 network
+    std::vector<float> w(2 * 16 * 16);
+    for (size_t i = 0; i < w.size(); ++i) w[i] = (float)(i % 97) / 128.0f;
+    io::saveCSV(dir + "w.csv", w);
+    const std::vector<tnn::half> packed = io::load_weights_as_packed_from_file<tnn::half, 16>(dir + "w.csv", 1, 16, 16);
+    CHECK(packed.size() == w.size());
+    bool same = true;
+    for (int m = 0; m < 2; ++m)
+        for (int k = 0; k < 16; ++k)
+            for (int n = 0; n < 16; ++n) same = same && (float)packed[m * 256 + toPackedLayoutCoord(k * 16 + n, 16, 16)] == w[m * 256 + k * 16 + n];
+    CHECK(same);
+}
+
 // ------------------------------------------------------------------------------------------- GPU cases
 
 template <typename T, int W> static void test_swiftnet(Activation act, Activation out_act, int L, size_t M, int in_w, int out_w, bool use_bias) {
@@ -618,6 +653,8 @@ int main(int argc, char **argv) {
     test_packed_coords();
     std::printf("json\n");
     test_json();
+    std::printf("io files\n");
+    test_io_files();
     if (!cpu_only) {
         tnn::abi_check(tnn_device_check());
         std::printf("swiftnet\n");

@@ -28,12 +28,13 @@ PEAK_HBM = 8000.0  # GB/s
 # HBM-side bytes per launch of each workload's dominant kernel at the default batch sizes, from rocprofv3 counter runs over this
 # file (FETCH_SIZE and WRITE_SIZE, one run each, scaled by what the same counter reads for the --copy-calibration kernel:
 # x2.000 and x1.000). The summaries with the commands are profiles/mlp_train_fused_kernel.*.txt, profiles/mlp_forward_kernel.*.txt,
-# profiles/grid_forward_kernel.*.txt and profiles/grid_mlp_inference_kernel.*.txt. Not measured live: counters need the profiler.
+# profiles/grid_forward_kernel.*.txt, profiles/grid_mlp_inference_kernel.*.txt and profiles/grid_backward_kernel.*.txt. Not measured live: counters need the profiler.
 MEASURED_TRAFFIC_BYTES = {
     ("train", 18): (57883.7 * 2.0 + 20488.0) * 1024,
     ("infer", 18): (16573.3 * 2.0 + 32768.7) * 1024,
     ("grid", 21): (6226188.0 * 2.0 + 262133.8) * 1024,
     ("grid_mlp", 21): (6641648.3 * 2.0 + 263928.2) * 1024,
+    ("grid_train", 18): (146433.7 * 2.0 + 731738.7) * 1024,  # the scatter kernel; its atomics count as 32-byte writes
 }
 
 
@@ -42,8 +43,10 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="train", choices=["train", "infer", "grid", "grid_mlp"])
+    ap.add_argument("--workload", default="train", choices=["train", "infer", "grid", "grid_mlp", "grid_train"])
     ap.add_argument("--batch-log2", type=int, default=None)
+    ap.add_argument("--packed-scatter", action="store_true",
+                    help="grid_train only: gradient table in fp16 with one packed atomic per feature pair (tnn_grid_backward_packed)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also launch a plain copy kernel (tnn_cast fp32 -> fp32, 256 MiB read + 256 MiB written per launch) so that "
@@ -146,6 +149,41 @@ def cpu_baseline_grid_mlp(oracle, cfg, w, budget_s=12.0):
     dt = time.perf_counter() - t0
     return {"value": M * k / dt, "unit": "points/s", "cores": oracle.num_threads(), "kind": "port",
             "sample": f"{k} passes of {M} points: encoding through the full 162 MiB table, then the 4-matrix network, OpenMP over points"}
+
+
+def cpu_baseline_grid_train(oracle, cfg, w, budget_s=12.0):
+    """Config 4's step on the host: encoding, network forward, L2 loss, network backward with dL/d(encoding), scatter into the
+    gradient table. (The two Adam updates are elementwise and left out.)"""
+    import numpy as np
+    from tolerances import FP16
+
+    rng = np.random.default_rng(0)
+    off, _, _ = oracle.grid_offsets(cfg["n_dims"], cfg["n_levels"], cfg["log2_hashmap_size"], cfg["base_resolution"], cfg["per_level_scale"])
+    n = int(off[-1]) * cfg["n_features_per_level"]
+    table = oracle.round(rng.uniform(-1e-4, 1e-4, n), FP16)
+    M = 1 << 14
+    x = rng.uniform(0, 1, (M, cfg["n_dims"])).astype(np.float32)
+    targets = np.zeros((M, 64), np.float32)
+    targets[:, :3] = rng.uniform(0, 1, (M, 3))
+    n_mats = w.shape[0]
+
+    def step():
+        enc = oracle.round(oracle.grid_forward(cfg, table, x, 64), FP16)
+        interm = oracle.mlp_forward_T(FP16, 64, n_mats, "relu", "none", w, enc)
+        _, grads = oracle.l2_loss(FP16, interm[-1], targets, 128.0)
+        _, _, d_enc = oracle.mlp_backward_T(FP16, 64, n_mats, "relu", "none", w, interm, grads, round_dw=False)
+        oracle.grid_backward(cfg, x, d_enc, n)
+
+    step()
+    t0 = time.perf_counter()
+    k = 0
+    while time.perf_counter() - t0 < budget_s:
+        step()
+        k += 1
+    dt = time.perf_counter() - t0
+    return {"value": M * k / dt, "unit": "samples/s", "cores": oracle.num_threads(), "kind": "port",
+            "sample": f"{k} steps of {M} points: encoding, network forward, L2, network backward, scatter into the 7.7 M-entry gradient "
+                      "table; OpenMP over points"}
 
 
 def main():
@@ -294,6 +332,99 @@ def main():
         }
         if oracle is not None:
             out["cpu_baseline"] = cpu_baseline_infer(oracle, W, n_mats)
+
+    elif args.workload == "grid_train":
+        # BASELINE config 4: 2-D hash grid -> w64 network with 2 hidden layers, 3 real outputs, one whole optimisation step:
+        # encoding, fused network step (forward, L2, backward, dL/d(encoding), Adam on the weights), scatter into the gradient
+        # table, Adam on the table's fp32 master with the fp16 table re-rounded
+        cfg = dict(n_dims=2, n_levels=16, n_features_per_level=2, log2_hashmap_size=19, base_resolution=16, per_level_scale=1.5)
+        W, n_hidden, n_out = 64, 2, 3
+        M = 1 << (args.batch_log2 or 18)
+        gd = t.grid_desc(cfg, FP16)
+        n = t.grid_n_params(gd)
+        gen = torch.Generator(device=t.dev).manual_seed(7)
+        table_master = torch.rand(n, device=t.dev, generator=gen) * 2e-4 - 1e-4
+        table = table_master.to(torch.float16)
+        mt, vt = torch.zeros_like(table_master), torch.zeros_like(table_master)
+        grad_table = torch.zeros(n, dtype=torch.float16 if args.packed_scatter else torch.float32, device=t.dev)
+        x = torch.rand((M, 2), device=t.dev, generator=gen)
+        targets = torch.zeros((M, W), device=t.dev)
+        targets[:, :n_out] = torch.rand((M, n_out), device=t.dev, generator=gen)
+        mdesc = t.mlp_desc(FP16, W, n_hidden, "relu", "none")
+        md = ctypes.byref(mdesc)
+        rng = np.random.default_rng(42)
+        lim = np.sqrt(6.0 / (2 * W))
+        w = rng.uniform(-lim, lim, (n_hidden + 1, W, W)).astype(np.float32)
+        w[0, 32:, :] = 0
+        w[-1, :, n_out:] = 0
+        master = t.pack(FP32, W, n_hidden + 1, torch.from_numpy(w.reshape(-1)).to(t.dev))
+        pf, pb = t.prepare_packed(mdesc, master, src_is_fp32=True)
+        mw, vw = torch.zeros_like(master), torch.zeros_like(master)
+        loss = torch.zeros(1, device=t.dev)
+        enc = torch.empty((M, W), dtype=torch.float16, device=t.dev)
+        d_enc = torch.empty_like(enc)
+        ws_bytes = lib.tnn_mlp_train_step_workspace_bytes(md, M)
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=t.dev)
+        # the loss of the config averages over the 3 real outputs, the fused step over the padded width: the factor W / 3 goes
+        # into the loss scale, which also keeps the fp16 gradients clear of the denormal range at this batch size
+        loss_scale = 128.0 * W / n_out * (M / 8192)
+        s = t.stream()
+        g = ctypes.byref(gd)
+        hyper = (1e-3, 0.9, 0.99, 1e-15)
+        k0, k1 = ev(), ev()
+
+        def step(i, time_scatter=False):
+            _lib.check(lib.tnn_grid_forward(g, ptr(x), ptr(table), ptr(enc), FP16, W, M, s))
+            _lib.check(lib.tnn_mlp_train_step_l2_adam(md, ptr(pf), ptr(pb), ptr(enc), ptr(targets), loss_scale, None, ptr(loss), ptr(master),
+                                                      ptr(mw), ptr(vw), i + 1, *hyper, None, ptr(d_enc), M, ptr(ws), ws_bytes, None, s))
+            if time_scatter:
+                k0.record()
+            if args.packed_scatter:
+                _lib.check(lib.tnn_grid_backward_packed(g, ptr(x), ptr(d_enc), FP16, W, ptr(grad_table), 1, M, s))
+            else:
+                _lib.check(lib.tnn_grid_backward(g, ptr(x), ptr(d_enc), FP16, W, ptr(grad_table), 1, M, s))
+            if time_scatter:
+                k1.record()
+            _lib.check(lib.tnn_adam_step(ptr(table_master), ptr(mt), ptr(vt), ptr(grad_table), FP16 if args.packed_scatter else FP32,
+                                         1.0 / loss_scale, n, i + 1, *hyper, ptr(table), FP16, s))
+
+        K = min(K, 50)
+        Wm = min(Wm, 5)
+        for i in range(Wm):
+            step(i)
+        torch.cuda.synchronize()
+        loss0 = float(loss.item()) * W / n_out  # mean over the real outputs
+        e0, e1 = ev(), ev()
+        e0.record()
+        for i in range(K):
+            step(Wm + i)
+        e1.record()
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1) / K
+        scatter_ms = 0.0
+        for i in range(10):  # the scatter (fill of the gradient table + atomics) on its own, outside the timed region
+            step(Wm + K + i, time_scatter=True)
+            torch.cuda.synchronize()
+            scatter_ms += k0.elapsed_time(k1) / 10
+        # algorithmic bytes of the scatter per point: coordinates + dL/d(encoding) row + read-modify-write of 16 levels x 4 corners x
+        # 2 features (4-byte gradients: 1096 B; 2-byte: 584 B)
+        gb = 2 if args.packed_scatter else 4
+        bpp = 8 + 32 * 2 + 16 * 4 * 2 * gb * 2
+        out = {
+            "metric": "hash-grid + fused-MLP training samples/s (2-D, 16x2, log2 19; w64, 2 hidden layers; batch 2^18; whole step with both Adam updates)",
+            "value": M / (ms * 1e-3), "unit": "samples/s", "n_gpus": 1, "steps": K, "warmup": Wm, "ms_per_step": ms,
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+            "config": {"workload": f"2-D hash-grid encoding + w64/2-hidden-layer network, one optimisation step, 2^{int(np.log2(M))} points "
+                                   f"(BASELINE config 4; gradient table {'fp16, packed atomics' if args.packed_scatter else 'fp32'})", "batch": M},
+            "roofline": {"bound": "hbm", "achieved": bpp * M / (scatter_ms * 1e-3) / 1e9, "peak": PEAK_HBM, "unit": "GB/s",
+                         "frac": bpp * M / (scatter_ms * 1e-3) / 1e9 / PEAK_HBM,
+                         "traffic": MEASURED_TRAFFIC_BYTES.get(("grid_train_packed" if args.packed_scatter else "grid_train", int(np.log2(M)))),
+                         "kernel": "grid_backward_kernel (with the fill of the gradient table in front of it)",
+                         "kernel_ms": scatter_ms, "algorithmic_bytes_per_launch": bpp * M},
+            "loss_first": loss0, "loss_last": float(loss.item()) * W / n_out,
+        }
+        if oracle is not None:
+            out["cpu_baseline"] = cpu_baseline_grid_train(oracle, cfg, oracle.round(w, FP16))
 
     else:
         cfg = dict(n_dims=3, n_levels=16, n_features_per_level=2, log2_hashmap_size=22, base_resolution=16, per_level_scale=1.447)

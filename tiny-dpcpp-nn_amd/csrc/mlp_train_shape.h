@@ -17,7 +17,7 @@ template <int W> struct TrainShape {
     static size_t lds_bytes(int n_mats) {
         const size_t stage = (size_t)WAVES * 2 * TILE_BYTES;
         const size_t reduce = (size_t)n_mats * W * W * 4; // end-of-kernel sum over the waves that share a tile
-        const size_t main = 2 * weight_bytes(n_mats) + stage;
+        const size_t main = 2 * weight_bytes(n_mats) + stage + 64; // + the arrival counters of the half-workgroups
         return main > reduce ? main : reduce;
     }
 };

@@ -30,7 +30,7 @@ PEAK_HBM = 8000.0  # GB/s
 # x2.000 and x1.000). The summaries with the commands are profiles/mlp_train_fused_kernel.*.txt, profiles/mlp_forward_kernel.*.txt,
 # profiles/grid_forward_kernel.*.txt, profiles/grid_mlp_inference_kernel.*.txt and profiles/grid_backward_kernel.*.txt. Not measured live: counters need the profiler.
 MEASURED_TRAFFIC_BYTES = {
-    ("train", 18): (57883.7 * 2.0 + 20488.0) * 1024,
+    ("train", 18): (56903.1 * 2.0 + 20488.0) * 1024,
     ("infer", 18): (16573.3 * 2.0 + 32768.7) * 1024,
     ("grid", 21): (6226188.0 * 2.0 + 262133.8) * 1024,
     ("grid_mlp", 21): (6641648.3 * 2.0 + 263928.2) * 1024,

@@ -86,7 +86,8 @@ class _module_function(torch.autograd.Function):
             doutput = torch.hstack((doutput, pad))
 
         batch_size = input.shape[0]
-        doutput = (doutput * loss_scale).contiguous()
+        # loss scaling: 1 for bf16, where the two passes over the gradient (here and after the kernels) are skipped
+        doutput = (doutput if loss_scale == 1.0 else doutput * loss_scale).contiguous()
         with torch.no_grad():
             if "encoding_config" in ctx.info:
                 input_grad = None
@@ -104,8 +105,10 @@ class _module_function(torch.autograd.Function):
                     if input_grad is not None:
                         input_grad = input_grad.reshape(batch_size, -1)
 
-        grad = None if grad is None else (grad / loss_scale).reshape(params.shape).to(params.dtype)
-        input_grad = None if input_grad is None else (input_grad / loss_scale)
+        if grad is not None:
+            grad = (grad if loss_scale == 1.0 else grad / loss_scale).reshape(params.shape).to(params.dtype)
+        if input_grad is not None and loss_scale != 1.0:
+            input_grad = input_grad / loss_scale
         # one entry per argument of forward
         return (None, input_grad, grad, None, None)
 

@@ -151,15 +151,17 @@ class Module(torch.nn.Module):
                 raise RuntimeError("Network has no parameters. Cannot set params")
             return
 
-        packed = params is None and self.name != "encoding"  # encoding parameters are never packed
-        if params is None:
+        pushing_own = params is None
+        packed = pushing_own and self.name != "encoding"  # encoding parameters are never packed
+        if pushing_own:
             params = self.params
         assert isinstance(params, torch.Tensor), "Params is not a torch.Tensor"
 
         self.tnn_module.set_params(params.detach().to(self.dtype).contiguous(), packed)
 
-        if not packed:
-            # keep the Python-side copy equal to what the native module holds (always the packed layout)
+        if not pushing_own:
+            # keep the Python-side copy equal to what the native module holds (networks: the packed layout). When the
+            # module's own `.params` were pushed the two already agree, and the copy back (a whole table for a grid) is skipped.
             self.params.data.copy_(self.get_params().reshape(self.params.shape))
 
     def get_params(self):

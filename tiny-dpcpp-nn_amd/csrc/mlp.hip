@@ -12,6 +12,7 @@
 // :443-487 (fp32 accumulate -> round to T -> activation; backward mask / sigmoid slope applied to
 // the fp32 accumulator before rounding).
 #include "mlp_tile.h"
+#include "mlp_train_shape.h"
 
 #include <cstdlib>
 
@@ -811,6 +812,10 @@ TNN_API int tnn_mlp_backward(const tnn_mlp_desc *desc, const void *d_prepared_bw
     float *partials = reinterpret_cast<float *>(base);
     void *deltas = d_interm_bwd ? d_interm_bwd : reinterpret_cast<void *>(base + partial_rounded);
     hipStream_t s = as_stream(stream);
+    // one kernel for deltas and weight gradients where the shape has it (width <= 64, up to 9 matrices); the deltas are
+    // then written only if the caller asked for them
+    rc = fused_backward(desc, d_prepared_bwd, d_dLdy, d_interm_fwd, d_interm_bwd, d_dW, dW_is_fp32, d_dLdx, M, partials, p.partial_bytes, s);
+    if (rc != TNN_ERR_UNSUPPORTED) return rc;
     TNN_DISPATCH_TW(desc, rc = (launch_backward<T_, W_>(desc, d_prepared_bwd, d_dLdy, d_interm_fwd, deltas, d_dLdx, M, s)));
     if (rc) return rc;
     TNN_DISPATCH_TW(desc, rc = (launch_dw<T_, W_>(desc, deltas, d_interm_fwd, d_dW, dW_is_fp32, M, partials, s)));

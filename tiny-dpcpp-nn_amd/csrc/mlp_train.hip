@@ -57,6 +57,13 @@ int fused_train_step(const tnn_mlp_desc *d, const void *wf, const void *wb, cons
     return fused_train_launch_fp16(d, p, wf, wb, x, targets, loss_scale, y, loss_sum, dW, dW_is_fp32, dx, M, partials, loss_partials, tail, s);
 }
 
+int fused_backward(const tnn_mlp_desc *d, const void *wb, const void *dLdy, const void *interm_fwd, void *interm_bwd, void *dW,
+                   int dW_is_fp32, void *dx, size_t M, float *partials, size_t partial_bytes, hipStream_t s) {
+    if (d->width > 64) return TNN_ERR_UNSUPPORTED;
+    if (d->dtype == TNN_BF16) return fused_backward_launch_bf16(d, wb, dLdy, interm_fwd, interm_bwd, dW, dW_is_fp32, dx, M, partials, partial_bytes, s);
+    return fused_backward_launch_fp16(d, wb, dLdy, interm_fwd, interm_bwd, dW, dW_is_fp32, dx, M, partials, partial_bytes, s);
+}
+
 // 0 when the shape has no fused kernel
 size_t fused_train_workspace_bytes(const tnn_mlp_desc *d, size_t M) {
     const FusedPlan p = fused_plan(d, M);

@@ -43,7 +43,7 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="train", choices=["train", "infer", "grid", "grid_mlp", "grid_train"])
+    ap.add_argument("--workload", default="train", choices=["train", "train_fb", "infer", "grid", "grid_mlp", "grid_train"])
     ap.add_argument("--batch-log2", type=int, default=None)
     ap.add_argument("--packed-scatter", action="store_true",
                     help="grid_train only: gradient table in fp16 with one packed atomic per feature pair (tnn_grid_backward_packed)")
@@ -213,7 +213,7 @@ def main():
     ev = lambda: torch.cuda.Event(enable_timing=True)
     out = {}
 
-    if args.workload in ("train", "infer"):
+    if args.workload in ("train", "train_fb", "infer"):
         W, n_hidden = 64, 4
         n_mats = n_hidden + 1
         M = 1 << (args.batch_log2 or 18)
@@ -298,6 +298,60 @@ def main():
             "mfma_frac_whole_step": flops / (ms * 1e-3) / 1e12 / PEAK_MFMA_BF16,
             "wall_ms_per_step": wall / K * 1e3,
             "loss_first": loss0, "loss_last": float(loss.item()),
+        }
+        if oracle is not None:
+            out["cpu_baseline"] = cpu_baseline_train(oracle, W, n_mats)
+
+    elif args.workload == "train_fb":
+        # The reference's own training step (Trainer::training_step, include/trainer.h:23-46): a forward pass that stores every
+        # activation, then a backward pass that returns the weight gradients, the deltas and dL/dx. No loss, no optimizer.
+        d = ctypes.byref(desc)
+        s = t.stream()
+        g = (torch.rand((M, W), device=t.dev, generator=gen) * 2 - 1).to(torch.bfloat16) / M
+        interm_f = torch.empty((n_mats + 1, M, W), dtype=torch.bfloat16, device=t.dev)
+        interm_b = torch.empty((n_mats, M, W), dtype=torch.bfloat16, device=t.dev)
+        dW = torch.empty(n_mats * W * W, dtype=torch.bfloat16, device=t.dev)
+        dX = torch.empty_like(x)
+        ws_bytes = lib.tnn_mlp_backward_workspace_bytes(d, M)
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=t.dev)
+        mid = ev()
+
+        def step(timed=False):
+            _lib.check(lib.tnn_mlp_forward(d, ptr(pf), ptr(x), ptr(interm_f), M, s))
+            if timed:
+                mid.record()
+            _lib.check(lib.tnn_mlp_backward(d, ptr(pb), ptr(g), ptr(interm_f), ptr(interm_b), ptr(dW), 0, ptr(dX), M, ptr(ws), ws_bytes, s))
+
+        for _ in range(Wm):
+            step()
+        torch.cuda.synchronize()
+        e0, e1 = ev(), ev()
+        e0.record()
+        for _ in range(K):
+            step()
+        e1.record()
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1) / K
+        bwd_ms = 0.0
+        for _ in range(10):  # the backward call on its own, outside the timed region
+            step(timed=True)
+            e1.record()
+            torch.cuda.synchronize()
+            bwd_ms += mid.elapsed_time(e1) / 10
+        flops = 3 * 2 * M * W * W * n_mats
+        # bytes of the backward call: dL/dy and n_mats activation matrices in, n_mats delta matrices and dL/dx out
+        bwd_bytes = (2 * n_mats + 2) * M * W * 2
+        out = {
+            "metric": "fused-MLP train & infer samples/s (w64, batch 2^18); % bf16 MFMA peak",
+            "value": M / (ms * 1e-3), "unit": "samples/s", "n_gpus": 1, "steps": K, "warmup": Wm, "ms_per_step": ms,
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+            "config": {"workload": f"training step as the reference's Trainer runs it: forward_pass with stored activations + backward_pass "
+                                   f"(deltas, dW, dL/dx), w64, 4 hidden layers, bf16, batch 2^{int(np.log2(M))}; no loss, no optimizer", "batch": M},
+            "roofline": {"bound": "hbm", "achieved": bwd_bytes / (bwd_ms * 1e-3) / 1e9, "peak": PEAK_HBM, "unit": "GB/s",
+                         "frac": bwd_bytes / (bwd_ms * 1e-3) / 1e9 / PEAK_HBM, "traffic": None,
+                         "kernel": "mlp_backward_fused_kernel (+ train_reduce_kernel)", "kernel_ms": bwd_ms,
+                         "algorithmic_bytes_per_launch": bwd_bytes},
+            "mfma_frac_whole_step": flops / (ms * 1e-3) / 1e12 / PEAK_MFMA_BF16,
         }
         if oracle is not None:
             out["cpu_baseline"] = cpu_baseline_train(oracle, W, n_mats)

@@ -22,7 +22,7 @@ def test_more_than_one_gpu_is_refused_with_a_message():
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("workload", ["train", "infer", "grid", "grid_mlp", "grid_train"])
+@pytest.mark.parametrize("workload", ["train", "train_fb", "infer", "grid", "grid_mlp", "grid_train"])
 def test_every_workload_prints_the_contract_line(workload):
     r = subprocess.run([sys.executable, BENCH, "--workload", workload, "--steps", "5", "--warmup", "2", "--no-cpu-baseline"],
                        capture_output=True, text=True, timeout=600)

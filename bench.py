@@ -32,6 +32,7 @@ PEAK_HBM = 8000.0  # GB/s
 MEASURED_TRAFFIC_BYTES = {
     ("train", 18): (56903.1 * 2.0 + 20488.0) * 1024,
     ("infer", 18): (16573.3 * 2.0 + 32768.7) * 1024,
+    ("train_fb", 18): (98684.3 * 2.0 + 217088.0) * 1024,  # the backward kernel
     ("grid", 21): (6226188.0 * 2.0 + 262133.8) * 1024,
     ("grid_mlp", 21): (6641648.3 * 2.0 + 263928.2) * 1024,
     ("grid_train", 18): (146433.7 * 2.0 + 731738.7) * 1024,  # the scatter kernel; its atomics count as 32-byte writes
@@ -348,7 +349,7 @@ def main():
             "config": {"workload": f"training step as the reference's Trainer runs it: forward_pass with stored activations + backward_pass "
                                    f"(deltas, dW, dL/dx), w64, 4 hidden layers, bf16, batch 2^{int(np.log2(M))}; no loss, no optimizer", "batch": M},
             "roofline": {"bound": "hbm", "achieved": bwd_bytes / (bwd_ms * 1e-3) / 1e9, "peak": PEAK_HBM, "unit": "GB/s",
-                         "frac": bwd_bytes / (bwd_ms * 1e-3) / 1e9 / PEAK_HBM, "traffic": None,
+                         "frac": bwd_bytes / (bwd_ms * 1e-3) / 1e9 / PEAK_HBM, "traffic": MEASURED_TRAFFIC_BYTES.get(("train_fb", int(np.log2(M)))),
                          "kernel": "mlp_backward_fused_kernel (+ train_reduce_kernel)", "kernel_ms": bwd_ms,
                          "algorithmic_bytes_per_launch": bwd_bytes},
             "mfma_frac_whole_step": flops / (ms * 1e-3) / 1e12 / PEAK_MFMA_BF16,

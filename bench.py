@@ -31,8 +31,8 @@ PEAK_HBM = 8000.0  # GB/s
 # profiles/grid_forward_kernel.*.txt, profiles/grid_mlp_inference_kernel.*.txt and profiles/grid_backward_kernel.*.txt. Not measured live: counters need the profiler.
 MEASURED_TRAFFIC_BYTES = {
     ("train", 18): (56903.1 * 2.0 + 20488.0) * 1024,
-    ("infer", 18): (16573.3 * 2.0 + 32768.7) * 1024,
-    ("train_fb", 18): (98684.3 * 2.0 + 217088.0) * 1024,  # the backward kernel
+    ("infer", 18): (16575.3 * 2.0 + 32768.0) * 1024,
+    ("train_fb", 18): (98600.4 * 2.0 + 217163.5) * 1024,  # the backward kernel
     ("grid", 21): (6226188.0 * 2.0 + 262133.8) * 1024,
     ("grid_mlp", 21): (6641648.3 * 2.0 + 263928.2) * 1024,
     ("grid_train", 18): (146433.7 * 2.0 + 731738.7) * 1024,  # the scatter kernel; its atomics count as 32-byte writes

@@ -61,7 +61,9 @@ __global__ void prepare_weights_kernel(const SRC *__restrict__ packed, T *__rest
 // ACT (hidden activation) is a compile-time constant so that the layer loop stays one basic block:
 // the fragments of the next matrix are requested from LDS before the current accumulators are
 // converted, and arrive while the conversion runs.
-template <typename T, int W, int ACT, bool STORE_INTERM, bool W_IN_LDS, int THREADS>
+// STAGED: every wave has a tile of LDS behind the weights and writes its rows through it (Tile::store_staged);
+// 2 = with the streaming hint.
+template <typename T, int W, int ACT, bool STORE_INTERM, bool W_IN_LDS, int THREADS, int STAGED = 0>
 __global__ void __launch_bounds__(THREADS, (THREADS == 512 && W <= 64) ? 4 : 1)
     mlp_forward_kernel(const typename Storage<T>::vec8 *__restrict__ wprep, const T *__restrict__ x, T *__restrict__ out,
                        int n_mats, int out_act, long long M) {
@@ -76,6 +78,16 @@ __global__ void __launch_bounds__(THREADS, (THREADS == 512 && W <= 64) ? 4 : 1)
     const long long n_tiles = (M + 31) / 32;
     const long long stride = (long long)gridDim.x * (blockDim.x >> 6);
     long long tile = (long long)blockIdx.x * (blockDim.x >> 6) + wave;
+    unsigned char *my_stage = smem_raw + (size_t)n_mats * (TL::NF * kWaveSize * sizeof(vec8)) + (size_t)wave * TL::TILE_BYTES;
+    unsigned int st_off[NK];
+    auto put = [&](const vec8(&r)[NK], T *dst, long long row, bool valid) __attribute__((always_inline)) {
+        if constexpr (STAGED != 0) {
+            TL::stage(r, my_stage, j, h);
+            TL::template store_staged<(STAGED == 2 ? kStreamingStore : 0)>(my_stage, lane, TL::rows_of(dst, M), st_off);
+        } else {
+            TL::store(r, dst, row, h, valid);
+        }
+    };
 
     // the first tile is requested before the weights are staged, so both latencies overlap
     vec8 cur[NK];
@@ -91,16 +103,17 @@ __global__ void __launch_bounds__(THREADS, (THREADS == 512 && W <= 64) ? 4 : 1)
         vec8 nxt[NK];
         if (next_tile < n_tiles) TL::load(nxt, x, next_tile * 32 + j, h, next_tile * 32 + j < M);
 
-        if (STORE_INTERM) TL::store(cur, out, row, h, valid);
+        if constexpr (STAGED != 0) TL::row_offsets(st_off, tile, lane, M);
+        if (STORE_INTERM) put(cur, out, row, valid);
         f32x16 acc[NI];
         for (int l = 0; l < n_mats - 1; ++l) {
             TL::template matmul<W_IN_LDS>(acc, cur, lds_w, wprep, l, lane);
             TL::template repack<ACT>(cur, acc);
-            if (STORE_INTERM) TL::store(cur, out + (size_t)(l + 1) * M * W, row, h, valid);
+            if (STORE_INTERM) put(cur, out + (size_t)(l + 1) * M * W, row, valid);
         }
         TL::template matmul<W_IN_LDS>(acc, cur, lds_w, wprep, n_mats - 1, lane);
         TL::repack_rt(cur, acc, out_act);
-        TL::store(cur, STORE_INTERM ? out + (size_t)n_mats * M * W : out, row, h, valid);
+        put(cur, STORE_INTERM ? out + (size_t)n_mats * M * W : out, row, valid);
 
         if (next_tile < n_tiles) {
 #pragma unroll
@@ -595,7 +608,30 @@ static int launch_forward_v(const tnn_mlp_desc *d, const void *wprep, const void
     if (in_lds && wbytes * per_cu > 160 * 1024) per_cu = (int)(160 * 1024 / wbytes);
     if (blocks > (long long)di.n_cu * per_cu) blocks = (long long)di.n_cu * per_cu;
     if (blocks < 1) blocks = 1;
-    if (in_lds) {
+    // Rows leave through a staged tile per wave (whole lines per store instruction) when that costs no workgroup per CU
+    // and the matrix fits 32-bit offsets; with the streaming hint for an inference result, and for activations whose
+    // volume exceeds the 256 MB of cache in front of the HBM (below that the backward pass finds them there).
+    const size_t staged_bytes = wbytes + (size_t)waves * Tile<T, W>::TILE_BYTES;
+    const bool staged = W <= 64 && in_lds && staged_bytes * per_cu <= 160 * 1024 &&
+                        (unsigned long long)M * W * sizeof(T) <= Tile<T, W>::kMaxBufferBytes;
+    const bool streaming = !STORE_INTERM || (unsigned long long)(n_mats + 1) * M * W * sizeof(T) > (256ull << 20);
+    if (staged) {
+        auto k1 = mlp_forward_kernel<T, W, ACT, STORE_INTERM, true, THREADS, (W <= 64 ? 1 : 0)>;
+        auto k2 = mlp_forward_kernel<T, W, ACT, STORE_INTERM, true, THREADS, (W <= 64 ? 2 : 0)>;
+        auto k = streaming ? k2 : k1;
+        // the reservation is a host round trip of several microseconds: once per kernel, device and size
+        static thread_local size_t reserved[2][16] = {};
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 16) return fail(TNN_ERR_HIP, "no usable HIP device");
+        if (staged_bytes > 48 * 1024 && reserved[streaming][dev] < staged_bytes) {
+            if (hipFuncSetAttribute(reinterpret_cast<const void *>(k), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    (int)staged_bytes) != hipSuccess)
+                return fail(TNN_ERR_HIP, "cannot reserve %zu bytes of LDS", staged_bytes);
+            reserved[streaming][dev] = staged_bytes;
+        }
+        TNN_LAUNCH(k, dim3((unsigned)blocks), dim3(THREADS), staged_bytes, s, (const vec8 *)wprep, (const T *)x,
+                           (T *)out, n_mats, d->output_activation, (long long)M);
+    } else if (in_lds) {
         auto k = mlp_forward_kernel<T, W, ACT, STORE_INTERM, true, THREADS>;
         if (wbytes > 48 * 1024 &&
             hipFuncSetAttribute(reinterpret_cast<const void *>(k), hipFuncAttributeMaxDynamicSharedMemorySize,

@@ -115,6 +115,10 @@ __device__ __forceinline__ typename Storage<T>::vec8 bwd_convert(const f32x16 &c
     return __builtin_bit_cast(typename Storage<T>::vec8, r);
 }
 
+// "nt" bit of a buffer store: the line is written through instead of staying dirty in L2 until the kernel ends. Only
+// with stores that cover whole 128-byte lines; with partial lines it costs more than it saves.
+constexpr int kStreamingStore = 2;
+
 template <typename T, int W> struct Tile {
     static constexpr int NK = W / 16;
     static constexpr int NI = (W + 31) / 32;
@@ -181,12 +185,14 @@ template <typename T, int W> struct Tile {
 #pragma unroll
         for (int kb = 0; kb < NK; ++kb) *reinterpret_cast<vec8 *>(tile_lds + j * PITCH + h * 16 + 32 * kb) = r[kb];
     }
+    // AUX: cache policy bits of the store; kStreamingStore marks data that this GPU does not read again soon.
+    template <int AUX = 0>
     static __device__ __forceinline__ void store_staged(const unsigned char *tile_lds, int lane, __amdgpu_buffer_rsrc_t rows,
                                                         const unsigned int (&o)[NK]) {
 #pragma unroll
         for (int i = 0; i < NK; ++i)
             __builtin_amdgcn_raw_buffer_store_b128(*reinterpret_cast<const u32x4 *>(tile_lds + (i * RPI + lane / LPR) * PITCH + (lane % LPR) * 16),
-                                                   rows, o[i], 0, 0);
+                                                   rows, o[i], 0, AUX);
     }
 
     static constexpr int NF = NI * NK; // weight fragments per matrix and lane

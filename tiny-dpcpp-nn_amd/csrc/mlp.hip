@@ -135,7 +135,9 @@ __global__ void __launch_bounds__(THREADS, (THREADS == 512 && W <= 64) ? 4 : 1)
 constexpr int kStreamThreads = 512;
 constexpr int kStreamTiles = 2;
 
-template <typename T, int W, int ACT, bool STORE_INTERM>
+// STAGED as in mlp_forward_kernel: 0 plain stores, 1 whole rows through a tile of LDS per wave (behind the two slots),
+// 2 the same with the streaming hint.
+template <typename T, int W, int ACT, bool STORE_INTERM, int STAGED = 0>
 __global__ void __launch_bounds__(kStreamThreads, 1)
     mlp_forward_stream_kernel(const typename Storage<T>::vec8 *__restrict__ wprep, const T *__restrict__ x, T *__restrict__ out,
                               int n_mats, int out_act, long long M) {
@@ -157,17 +159,28 @@ __global__ void __launch_bounds__(kStreamThreads, 1)
 #pragma unroll
     for (int i = 0; i < SHARE; ++i) lds[threadIdx.x + kStreamThreads * i] = wprep[threadIdx.x + kStreamThreads * i];
     int b = 0; // slot that holds the matrix of the layer about to run
+    unsigned char *my_stage = smem_raw + 2 * per_mat * sizeof(vec8) + (size_t)wave * TL::TILE_BYTES;
 
     for (long long r = blockIdx.x; r < n_rounds; r += gridDim.x) {
         long long row[R];
         bool valid[R];
         vec8 cur[R][NK];
+        unsigned int st_off[R][NK];
+        auto put = [&](int t, T *dst) __attribute__((always_inline)) {
+            if constexpr (STAGED != 0) {
+                TL::stage(cur[t], my_stage, j, h);
+                TL::template store_staged<(STAGED == 2 ? kStreamingStore : 0)>(my_stage, lane, TL::rows_of(dst, M), st_off[t]);
+            } else {
+                TL::store(cur[t], dst, row[t], h, valid[t]);
+            }
+        };
 #pragma unroll
         for (int t = 0; t < R; ++t) {
             row[t] = r * ROUND + (wave * R + t) * 32 + j;
             valid[t] = row[t] < M;
+            if constexpr (STAGED != 0) TL::row_offsets(st_off[t], r * (ROUND / 32) + wave * R + t, lane, M);
             TL::load(cur[t], x, row[t], h, valid[t]);
-            if (STORE_INTERM) TL::store(cur[t], out, row[t], h, valid[t]);
+            if (STORE_INTERM) put(t, out);
         }
         const bool more_rounds = r + gridDim.x < n_rounds;
         for (int l = 0; l < n_mats; ++l) {
@@ -202,10 +215,10 @@ __global__ void __launch_bounds__(kStreamThreads, 1)
             for (int t = 0; t < R; ++t) {
                 if (!last) {
                     TL::template repack<ACT>(cur[t], acc[t]);
-                    if (STORE_INTERM) TL::store(cur[t], out + (size_t)(l + 1) * M * W, row[t], h, valid[t]);
+                    if (STORE_INTERM) put(t, out + (size_t)(l + 1) * M * W);
                 } else {
                     TL::repack_rt(cur[t], acc[t], out_act);
-                    TL::store(cur[t], STORE_INTERM ? out + (size_t)n_mats * M * W : out, row[t], h, valid[t]);
+                    put(t, STORE_INTERM ? out + (size_t)n_mats * M * W : out);
                 }
             }
             b ^= 1;
@@ -589,15 +602,25 @@ static int launch_forward_v(const tnn_mlp_desc *d, const void *wprep, const void
     if (!di.ok) return fail(TNN_ERR_HIP, "no usable HIP device");
     const bool in_lds = wbytes <= kLdsBudget;
     if constexpr (W == 128) {
-        if (!in_lds) { // stream the matrices through LDS, one layer at a time
+        // also when the activations are stored and the weights would fit: the staging tiles of the whole-row stores do not
+        // fit beside 128 KiB of weights, and the stores are what that pass is bound by (4 matrices: 442 -> 239 us at 2^20
+        // rows, 124 -> 68 us at 2^18, no difference at 2^16, 1-3 us slower below)
+        if (!in_lds || (STORE_INTERM && M >= 65536)) { // stream the matrices through LDS, one layer at a time
             constexpr size_t lds = 2 * (size_t)Tile<T, W>::NI * Tile<T, W>::NK * kWaveSize * sizeof(vec8);
             constexpr long long round = (kStreamThreads / 64) * kStreamTiles * 32;
             long long g = ((long long)M + round - 1) / round;
             if (g > di.n_cu) g = di.n_cu;
-            auto k = mlp_forward_stream_kernel<T, W, ACT, STORE_INTERM>;
-            if (hipFuncSetAttribute(reinterpret_cast<const void *>(k), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
-                return fail(TNN_ERR_HIP, "cannot reserve %zu bytes of LDS", lds);
-            TNN_LAUNCH(k, dim3((unsigned)g), dim3(kStreamThreads), lds, s, (const vec8 *)wprep, (const T *)x, (T *)out, n_mats,
+            const bool fits32 = (unsigned long long)M * W * sizeof(T) <= Tile<T, W>::kMaxBufferBytes;
+            const bool streaming = !STORE_INTERM || (unsigned long long)(n_mats + 1) * M * W * sizeof(T) > (256ull << 20);
+            const size_t lds_staged = lds + (kStreamThreads / 64) * (size_t)Tile<T, W>::TILE_BYTES;
+            auto k0 = mlp_forward_stream_kernel<T, W, ACT, STORE_INTERM, 0>;
+            auto k1 = mlp_forward_stream_kernel<T, W, ACT, STORE_INTERM, 1>;
+            auto k2 = mlp_forward_stream_kernel<T, W, ACT, STORE_INTERM, 2>;
+            auto k = !fits32 ? k0 : (streaming ? k2 : k1);
+            const size_t lds_k = fits32 ? lds_staged : lds;
+            if (hipFuncSetAttribute(reinterpret_cast<const void *>(k), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_k) != hipSuccess)
+                return fail(TNN_ERR_HIP, "cannot reserve %zu bytes of LDS", lds_k);
+            TNN_LAUNCH(k, dim3((unsigned)g), dim3(kStreamThreads), lds_k, s, (const vec8 *)wprep, (const T *)x, (T *)out, n_mats,
                        d->output_activation, (long long)M);
             return check_launch("mlp_forward_stream_kernel");
         }

@@ -261,11 +261,12 @@ template <typename T, int WIDTH> class NetworkModule : public Module {
         if (batch_size == 0) return torch::empty({0, out_w}, torch::TensorOptions().dtype(torch_type<T>::dtype).device(device()));
         DeviceMatrixView<T> input_dm(batch_size, network_.get_input_width(), network_.get_input_width(),
                                      reinterpret_cast<T *>(input_tensor.data_ptr()));
-        this->AllocateWorkspace(batch_size);
-        DeviceMatricesView<T> output_network(1, batch_size, network_.get_output_width(), 0, 0, 0, 0, interm_forw_ptr_);
+        // the kernel writes the tensor that is handed back: a fresh allocation, as the reference's clone is, without the copy
+        torch::Tensor output = torch::empty({(int64_t)batch_size, out_w}, torch::TensorOptions().dtype(torch_type<T>::dtype).device(device()));
+        DeviceMatricesView<T> output_network(1, batch_size, network_.get_output_width(), 0, 0, 0, 0, reinterpret_cast<T *>(output.data_ptr()));
         network_.inference(input_dm, output_network, {});
         this->finish();
-        return fromDevice<T>(interm_forw_ptr_, {(int64_t)batch_size, out_w});
+        return output;
     }
 
     bool can_fuse_encoding(const Module &encoding) const override {
@@ -285,11 +286,11 @@ template <typename T, int WIDTH> class NetworkModule : public Module {
         const size_t batch_size = positions.sizes()[0];
         const int64_t out_w = network_.get_output_width();
         if (batch_size == 0) return torch::empty({0, out_w}, torch::TensorOptions().dtype(torch_type<T>::dtype).device(device()));
-        this->AllocateWorkspace(batch_size);
-        DeviceMatricesView<T> output_network(1, batch_size, network_.get_output_width(), 0, 0, 0, 0, interm_forw_ptr_);
+        torch::Tensor output = torch::empty({(int64_t)batch_size, out_w}, torch::TensorOptions().dtype(torch_type<T>::dtype).device(device()));
+        DeviceMatricesView<T> output_network(1, batch_size, network_.get_output_width(), 0, 0, 0, 0, reinterpret_cast<T *>(output.data_ptr()));
         network_.inference_with_grid(*grid, encoding.grid_table(), positions.data_ptr<float>(), batch_size, output_network);
         this->finish();
-        return fromDevice<T>(interm_forw_ptr_, {(int64_t)batch_size, out_w});
+        return output;
     }
 
     torch::Tensor forward_pass(const torch::Tensor &input_tensor) override {
@@ -330,7 +331,13 @@ template <typename T, int WIDTH> class NetworkModule : public Module {
         DeviceMatricesView<T> interm_bwd(network_.get_n_hidden_layers() + 1, batch_size, network_.get_input_width(), batch_size,
                                          network_.get_network_width(), batch_size, network_.get_output_width(), interm_backw_ptr_);
         DeviceMatricesView<T> interm_fwd = ForwardViews(batch_size);
-        DeviceMatrixView<T> dL_dinput(batch_size, network_.get_input_width(), network_.get_input_width(), dL_dinput_ptr_);
+        // dL/dinput goes straight into the tensor that is handed back
+        torch::Tensor input_grad;
+        if (get_dl_dinput)
+            input_grad = torch::empty({(int64_t)(batch_size * network_.get_input_width()), 1},
+                                      torch::TensorOptions().dtype(torch_type<T>::dtype).device(device()));
+        DeviceMatrixView<T> dL_dinput(batch_size, network_.get_input_width(), network_.get_input_width(),
+                                      get_dl_dinput ? reinterpret_cast<T *>(input_grad.data_ptr()) : dL_dinput_ptr_);
 
         network_.backward_pass(dL_doutput, net_gradients_.GetViews(), interm_bwd, interm_fwd, {}, get_dl_dinput ? &dL_dinput : nullptr);
         this->finish();
@@ -344,8 +351,6 @@ template <typename T, int WIDTH> class NetworkModule : public Module {
             result = &net_gradients_packed_;
         }
 
-        torch::Tensor input_grad;
-        if (get_dl_dinput) input_grad = fromDevice<T>(dL_dinput.GetPointer(), {(int64_t)dL_dinput.nelements(), 1});
         return {input_grad, fromDevice<T>(result->GetViews().GetMatrixPointer(0), {(int64_t)result->nelements(), 1})};
     }
 

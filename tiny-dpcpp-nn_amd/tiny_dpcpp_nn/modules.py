@@ -100,8 +100,9 @@ class _module_function(torch.autograd.Function):
                 if batch_size == 0:
                     input_grad, grad = torch.zeros_like(input), torch.zeros_like(params)
                 else:
-                    # pack the gradient into the parameter layout, and get dL/dinput
-                    input_grad, grad = ctx.native_tnn_module.bwd_no_encoding_grad(doutput, True, True)
+                    # pack the gradient into the parameter layout; dL/dinput only when autograd asks for it (the product
+                    # with the first matrix and a batch-sized store otherwise serve nobody)
+                    input_grad, grad = ctx.native_tnn_module.bwd_no_encoding_grad(doutput, True, bool(ctx.needs_input_grad[1]))
                     if input_grad is not None:
                         input_grad = input_grad.reshape(batch_size, -1)
 
@@ -157,7 +158,10 @@ class Module(torch.nn.Module):
             params = self.params
         assert isinstance(params, torch.Tensor), "Params is not a torch.Tensor"
 
-        self.tnn_module.set_params(params.detach().to(self.dtype).contiguous(), packed)
+        pushed = params.detach()
+        if not (pushed.is_cuda and pushed.dtype in (torch.float32, torch.float16, torch.bfloat16) and self.name != "encoding"):
+            pushed = pushed.to(self.dtype)  # a network on the GPU converts to its own type itself, in the kernel that copies
+        self.tnn_module.set_params(pushed.contiguous(), packed)
 
         if not pushing_own:
             # keep the Python-side copy equal to what the native module holds (networks: the packed layout). When the

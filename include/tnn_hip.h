@@ -260,7 +260,8 @@ int tnn_grid_backward(const tnn_grid_desc *desc, const float *d_x, const void *d
                       uint32_t padded_width, float *d_grad_table, int overwrite, size_t M, tnn_stream_t stream);
 
 /* The same scatter into an fp16 gradient table, two features of an entry per packed atomic (global_atomic_pk_add_f16): half
- * as many atomic operations as the fp32 route, which is what bounds the pass. No counterpart in the reference, whose
+ * as many atomic operations as the fp32 route and half the gradient table; the same number of 32-byte requests at the memory
+ * side, which is what bounds the pass, so about the same time. No counterpart in the reference, whose
  * gradients are float (grad_t, include/encodings/grid.h:586, "we don't have atomics for half precision",
  * dpcpp_bindings/tiny_dpcpp_nn/modules.py:320-324); it is what tiny-cuda-nn does for half-precision grids. Sums are
  * rounded to fp16 at every addition: scale dL/dy (loss scale) so that contributions stay clear of fp16's denormal range.

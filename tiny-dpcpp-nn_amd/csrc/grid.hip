@@ -121,7 +121,7 @@ struct BackwardPlan {
     uint32_t n_small;          // levels whose whole gradient slice fits the LDS budget
     uint32_t small_blocks;     // workgroups per such level, each takes `chunk` consecutive points
     uint32_t chunk;
-    uint32_t big_blocks;       // workgroups per other level, one point per thread
+    uint32_t big_blocks;       // workgroups per other level, a group of lanes per point
     uint8_t small_level[TNN_GRID_MAX_LEVELS];
     uint8_t big_level[TNN_GRID_MAX_LEVELS];
 };
@@ -175,12 +175,16 @@ template <int F> __device__ __forceinline__ void add_entry(fp16_t *entry, const 
     }
 }
 
+// Lanes over the features of one entry on the direct route: one per value for an fp32 table, one per packed pair for fp16.
+template <int F, typename GT> struct BackwardLanes { static constexpr int FL = F; };
+template <int F> struct BackwardLanes<F, fp16_t> { static constexpr int FL = F / 2; };
+
 // Scatter-add of dL/dy into the gradient table (include/encodings/grid.h:137-245 of the reference: float atomics,
 // order not defined). Two routes inside one launch:
 //   * small levels (the coarse ones, where every point of the batch lands on a few hundred entries and global
 //     atomics queue up on the same addresses): a workgroup adds the contributions of a chunk of points into a
 //     private copy of the level in LDS and then issues one global atomic per touched entry;
-//   * the other levels: one thread per (point, level), atomics straight to the table; workgroups of one level
+//   * the other levels: a group of lanes per (point, level), atomics straight to the table; workgroups of one level
 //     are dispatched together, so its slice of the table is the hot one in L2.
 template <int D, int F, typename G, typename GT>
 __global__ void __launch_bounds__(kGridThreads)
@@ -223,24 +227,53 @@ __global__ void __launch_bounds__(kGridThreads)
         }
         return;
     }
+    // A group of 2 * FL neighbouring lanes owns one (point, level): lane (dx, fl) adds feature fl (fp16 table: the pair of
+    // features fl) of the corners on side dx of the cell along the first dimension. The memory side retires atomic
+    // requests per 32-byte sector, about 20 * 10^9 a second, however many lanes of one instruction fall into the sector:
+    // the features of an entry always do, and the two corners along the first dimension are neighbouring entries
+    // wherever that dimension enters the index unhashed or the hash leaves it in the low bits.
+    constexpr int FL = BackwardLanes<F, GT>::FL, LPI = 2 * FL;
     const uint32_t b = blockIdx.x - n_small_blocks;
     const uint32_t l = bp.big_level[b / bp.big_blocks];
-    const long long i = (long long)(b % bp.big_blocks) * kGridThreads + threadIdx.x;
+    const long long i = (long long)(b % bp.big_blocks) * (kGridThreads / LPI) + threadIdx.x / LPI;
     if (i >= M) return;
+    const int dx = (threadIdx.x % LPI) / FL, fl = threadIdx.x % FL;
     float x[D];
 #pragma unroll
     for (int d = 0; d < D; ++d) x[d] = xin[i * D + d];
-    float gy[F];
+    constexpr int FV = F / FL; // values per lane: 1 (fp32 table) or 2 (fp16 table)
+    float gy[FV];
 #pragma unroll
-    for (int f = 0; f < F; ++f) gy[f] = (float)dLdy[i * gp.padded_width + l * F + f];
-    GT *g = grad + (size_t)lv.offset[l] * F;
-    for_each_corner<D>(x, lv.scale[l], lv.size[l], lv.resolution[l], lv.flags[l], gp.hash_type, gp.interpolation,
-                       [&](uint32_t idx, float w) {
-                           float v[F];
+    for (int f = 0; f < FV; ++f) gy[f] = (float)dLdy[i * gp.padded_width + l * F + fl * FV + f];
+    GT *g = grad + (size_t)lv.offset[l] * F + fl * FV;
+    const uint32_t size = lv.size[l], res = lv.resolution[l], flags = lv.flags[l];
+    uint32_t cell[D];
+    float frac[D];
+    cell_of<D>(x, lv.scale[l], gp.interpolation, cell, frac);
+    if (gp.interpolation == TNN_INTERP_NEAREST) {
+        if (dx == 0) add_entry<FV>(g + (size_t)level_index<D>(cell, size, res, flags, gp.hash_type) * F, gy);
+        return;
+    }
 #pragma unroll
-                           for (int f = 0; f < F; ++f) v[f] = w * gy[f];
-                           add_entry<F>(g + (size_t)idx * F, v);
-                       });
+    for (int rest = 0; rest < (1 << (D - 1)); ++rest) {
+        const int c = 2 * rest + dx; // same corner numbering and weight product as for_each_corner
+        float weight = 1.0f;
+        uint32_t loc[D];
+#pragma unroll
+        for (int d = 0; d < D; ++d) {
+            if ((c & (1 << d)) == 0) {
+                weight *= 1 - frac[d];
+                loc[d] = cell[d];
+            } else {
+                weight *= frac[d];
+                loc[d] = cell[d] + 1;
+            }
+        }
+        float v[FV];
+#pragma unroll
+        for (int f = 0; f < FV; ++f) v[f] = weight * gy[f];
+        add_entry<FV>(g + (size_t)level_index<D>(loc, size, res, flags, gp.hash_type) * F, v);
+    }
 }
 
 __global__ void fill_zero_kernel(float4 *__restrict__ p, size_t n4, float *__restrict__ tail, size_t n_tail) {
@@ -300,7 +333,8 @@ static int launch_grid_backward_g(const GridLevels &lv, const GridParams &gp, co
     BackwardPlan bp{};
     bp.chunk = kPrivateChunk;
     bp.small_blocks = (uint32_t)((M + bp.chunk - 1) / bp.chunk);
-    bp.big_blocks = (uint32_t)((M + kGridThreads - 1) / kGridThreads);
+    constexpr int per_block = kGridThreads / (2 * BackwardLanes<F, TAB>::FL); // (point, level) pairs per workgroup on the direct route
+    bp.big_blocks = (uint32_t)((M + per_block - 1) / per_block);
     const size_t per_chunk = (M < bp.chunk ? M : (size_t)bp.chunk) << (gp.interpolation == TNN_INTERP_NEAREST ? 0 : D);
     uint32_t n_big = 0, lds_bytes = 0;
     for (uint32_t l = 0; l < gp.n_levels; ++l) {

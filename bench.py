@@ -42,8 +42,10 @@ MEASURED_TRAFFIC_BYTES = {
 def parse():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=20)
+    # a step takes 15-60 us: the first few hundred run while the clocks still ramp up (58.9 us per training step over 200 steps
+    # after 20, 54.0 over 1000 after 200, 53.6 over 2000 after 500), so the defaults time a second of steady state at most
+    ap.add_argument("--steps", type=int, default=1000)
+    ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--workload", default="train", choices=["train", "train_fb", "infer", "grid", "grid_mlp", "grid_train"])
     ap.add_argument("--batch-log2", type=int, default=None)
     ap.add_argument("--packed-scatter", action="store_true",

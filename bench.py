@@ -30,12 +30,12 @@ PEAK_HBM = 8000.0  # GB/s
 # x2.000 and x1.000). The summaries with the commands are profiles/mlp_train_fused_kernel.*.txt, profiles/mlp_forward_kernel.*.txt,
 # profiles/grid_forward_kernel.*.txt, profiles/grid_mlp_inference_kernel.*.txt and profiles/grid_backward_kernel.*.txt. Not measured live: counters need the profiler.
 MEASURED_TRAFFIC_BYTES = {
-    ("train", 18): (56903.1 * 2.0 + 20488.0) * 1024,
-    ("infer", 18): (16575.3 * 2.0 + 32768.0) * 1024,
-    ("train_fb", 18): (98600.4 * 2.0 + 217163.5) * 1024,  # the backward kernel
-    ("grid", 21): (6226188.0 * 2.0 + 262133.8) * 1024,
-    ("grid_mlp", 21): (6641648.3 * 2.0 + 263928.2) * 1024,
-    ("grid_train", 18): (211577.6 * 2.0 + 236762.7) * 1024,  # the scatter kernel; an atomic request counts as a 32-byte write
+    ("train", 18): (56937.8 * 2.0 + 20488.0) * 1024,
+    ("infer", 18): (16575.2 * 2.0 + 32768.0) * 1024,
+    ("train_fb", 18): (98600.2 * 2.0 + 217143.4) * 1024,  # the backward kernel
+    ("grid", 21): (6211700.1 * 2.0 + 262135.3) * 1024,
+    ("grid_mlp", 21): (6637904.7 * 2.0 + 263960.6) * 1024,
+    ("grid_train", 18): (211580.8 * 2.0 + 236762.7) * 1024,  # the scatter kernel; an atomic request counts as a 32-byte write
 }
 
 

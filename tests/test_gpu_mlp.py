@@ -198,6 +198,63 @@ def test_argument_checks(tnn):
     assert b"workspace" in tnn.lib.tnn_last_error()
 
 
+@pytest.mark.parametrize("dtype,W,n_hidden,M", [
+    (FP16, 128, 2, (1 << 16) + 24),  # width 128, few matrices, activations stored: the route that streams the matrices through LDS
+    (BF16, 64, 4, (1 << 20) + 8),    # 805 MB of activations: whole-row stores with the streaming hint
+    (FP16, 32, 4, (1 << 18) + 40),   # two rows per 128-byte line
+    (FP16, 16, 2, (1 << 18) + 8),    # four rows per line
+])
+def test_forward_store_routes_at_large_batches(tnn, oracle, dtype, W, n_hidden, M):
+    """The row stores of forward and inference take different routes with the batch size and the shape (plain, through a
+    staged tile, with or without the streaming hint). Rows are independent, so the first and the last 96 rows of a large,
+    ragged batch are compared with the oracle, matrix by matrix, and the two calls with each other over the whole batch."""
+    import torch
+    from gpu_harness import TORCH_DT
+    n_mats = n_hidden + 1
+    w = oracle.round(xavier(W, n_mats, 5), dtype)
+    gen = torch.Generator(device=tnn.dev).manual_seed(9)
+    xt = (torch.rand((M, W), device=tnn.dev, generator=gen) * 2 - 1).to(TORCH_DT[dtype])
+    desc = tnn.mlp_desc(dtype, W, n_hidden, "relu", "none")
+    _, pf, _ = tnn.prepare(desc, w)
+    interm_t = tnn.forward(desc, pf, xt)  # pre-filled with NaN by the harness
+    y_t = tnn.inference(desc, pf, xt)
+    assert not torch.isnan(interm_t).any(), "rows left unwritten"
+    assert torch.equal(interm_t[n_mats], y_t), "forward and inference disagree"
+    assert torch.equal(interm_t[0], xt), "interm_fwd[0] is not the input"
+    for rows in (slice(0, 96), slice(M - 96, M)):
+        ref = oracle.mlp_forward_T(dtype, W, n_mats, "relu", "none", w, tnn.host(xt[rows]))
+        for l in range(1, n_mats + 1):
+            assert_propagated(tnn.host(interm_t[l][rows]), ref[l], dtype, f"interm_fwd[{l}] rows {rows}")
+
+
+@pytest.mark.parametrize("dtype,W,n_hidden,M", [(BF16, 64, 4, (1 << 18) + 40), (FP16, 32, 2, (1 << 18) + 8), (FP16, 16, 2, (1 << 18) + 24)])
+def test_backward_store_route_at_large_batch(tnn, oracle, dtype, W, n_hidden, M):
+    """The fused backward writes its deltas and dL/dx as whole rows from staged tiles, through range-checked buffer stores.
+    Large ragged batch: nothing left unwritten, first and last rows against the oracle, and the weight gradients against
+    the product of the deltas and activations the GPU itself holds (fp64 on the device)."""
+    import torch
+    from gpu_harness import TORCH_DT
+    n_mats = n_hidden + 1
+    ls = 128.0 if dtype == FP16 else 1.0
+    w = oracle.round(xavier(W, n_mats, 8), dtype)
+    gen = torch.Generator(device=tnn.dev).manual_seed(10)
+    xt = (torch.rand((M, W), device=tnn.dev, generator=gen) * 2 - 1).to(TORCH_DT[dtype])
+    gt = ((torch.rand((M, W), device=tnn.dev, generator=gen) * 2 - 1) * (ls / M)).to(TORCH_DT[dtype])
+    desc = tnn.mlp_desc(dtype, W, n_hidden, "relu", "none")
+    _, pf, pb = tnn.prepare(desc, w)
+    interm_t = tnn.forward(desc, pf, xt)
+    ib, dW, dX = tnn.backward(desc, pb, gt, interm_t, dw_fp32=True)  # outputs pre-filled with NaN by the harness
+    assert not torch.isnan(ib).any() and not torch.isnan(dX).any() and not torch.isnan(dW).any()
+    for rows in (slice(0, 96), slice(M - 96, M)):
+        rib, _, rdX = oracle.mlp_backward_T(dtype, W, n_mats, "relu", "none", w, tnn.host(interm_t[:, rows]), tnn.host(gt[rows]), round_dw=False)
+        for l in range(n_mats):
+            assert_propagated(tnn.host(ib[l][rows]), rib[l], dtype, f"delta[{l}] rows {rows}", scale=ls / M)
+        assert_propagated(tnn.host(dX[rows]), rdX, dtype, f"dL/dx rows {rows}", scale=ls / M)
+    for l in range(n_mats):
+        exact = (ib[l].double().T @ interm_t[l].double()).cpu().numpy()
+        assert_close(tnn.host(dW[l]), exact, dtype, f"dW[{l}] from the GPU's own deltas", scale=ls)
+
+
 def test_baseline_config_1_full_size(tnn, oracle):
     """BASELINE config 1: w64, 4 hidden layers, bf16, ReLU / linear, batch 2^17, compared row for row."""
     dtype, W, n_hidden, M = BF16, 64, 4, 1 << 17

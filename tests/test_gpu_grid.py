@@ -78,10 +78,12 @@ def test_forward_values(tnn, oracle, cfg, param_dtype, out_dtype):
 
 
 @pytest.mark.parametrize("cfg", [CFG4, CFG5, dict(CFG4, interpolation="Smoothstep"), dict(CFG4, interpolation="Nearest"),
-                                 dict(CFG5, n_features_per_level=4, n_levels=8), dict(CFG4, n_features_per_level=1), dict(CFG4, n_features_per_level=8, n_levels=4)])
+                                 dict(CFG5, n_features_per_level=4, n_levels=8), dict(CFG4, n_features_per_level=1), dict(CFG4, n_features_per_level=8, n_levels=4),
+                                 dict(CFG4, grid_type="Dense", n_levels=7), dict(CFG5, grid_type="Tiled", n_levels=6, log2_hashmap_size=15),
+                                 dict(CFG5, hash="Prime", log2_hashmap_size=14, n_features_per_level=1)])
 def test_forward_backward_variants(tnn, oracle, cfg):
     rng = np.random.default_rng(13)
-    M = 2048
+    M = 2011  # no multiple of the (point, level) pairs a workgroup of the backward takes, whatever the feature count
     F, L = cfg["n_features_per_level"], cfg["n_levels"]
     pw = L * F + 8
     x = rng.uniform(0, 1, (M, cfg["n_dims"])).astype(np.float32)

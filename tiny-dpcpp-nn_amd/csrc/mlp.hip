@@ -602,10 +602,11 @@ static int launch_forward_v(const tnn_mlp_desc *d, const void *wprep, const void
     if (!di.ok) return fail(TNN_ERR_HIP, "no usable HIP device");
     const bool in_lds = wbytes <= kLdsBudget;
     if constexpr (W == 128) {
-        // also when the activations are stored and the weights would fit: the staging tiles of the whole-row stores do not
-        // fit beside 128 KiB of weights, and the stores are what that pass is bound by (4 matrices: 442 -> 239 us at 2^20
-        // rows, 124 -> 68 us at 2^18, no difference at 2^16, 1-3 us slower below)
-        if (!in_lds || (STORE_INTERM && M >= 65536)) { // stream the matrices through LDS, one layer at a time
+        // also for large batches when the weights would fit: the staging tiles of the whole-row stores do not fit beside
+        // 128 KiB of weights, and the stores are what these passes are bound by (forward with stored activations, 4 matrices:
+        // 442 -> 239 us at 2^20 rows, 124 -> 68 us at 2^18, no difference at 2^16, 1-3 us slower below; inference, 4 matrices:
+        // 197 -> 182 us at 2^20 rows, 2 matrices: 143 -> 105 us)
+        if (!in_lds || M >= 65536) { // stream the matrices through LDS, one layer at a time
             constexpr size_t lds = 2 * (size_t)Tile<T, W>::NI * Tile<T, W>::NK * kWaveSize * sizeof(vec8);
             constexpr long long round = (kStreamThreads / 64) * kStreamTiles * 32;
             long long g = ((long long)M + round - 1) / round;

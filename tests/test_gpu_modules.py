@@ -150,6 +150,12 @@ def test_network_forward_and_gradients(tcnn, oracle, dtype, width, n_hidden, n_i
         err = np.linalg.norm((got - ref).ravel()) / np.linalg.norm(ref.ravel())
         assert err <= bar, f"{what}: relative Frobenius error {err:g} vs fp32 autograd"
 
+    # an input that asks for no gradient: the backward leaves dL/dinput out, the parameter gradient is the same
+    grad_with_dx = net.params.grad.clone()
+    net.params.grad = None
+    net(x.to(DEVICE)).backward(g.to(DEVICE))
+    assert torch.equal(net.params.grad, grad_with_dx)
+
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 def test_set_params_constant(tcnn, dtype):

@@ -134,11 +134,12 @@ template <typename T> class EncodingModule : public Module {
         if (batch_size == 0) return torch::empty({0, (int64_t)out_w}, torch::TensorOptions().dtype(torch_type<T>::dtype).device(device()));
 
         DeviceMatrixView<float> input_dmv(batch_size, encoding_->get_input_width(), encoding_->get_input_width(), input_tensor.data_ptr<float>());
-        this->AllocateWorkspace(batch_size);
-        DeviceMatrixView<T> output_encoding(batch_size, out_w, out_w, output_encoding_ptr_);
+        // the kernel writes the tensor that is handed back (a fresh allocation as the reference's clone is, without the copy)
+        torch::Tensor output = torch::empty({(int64_t)batch_size, (int64_t)out_w}, torch::TensorOptions().dtype(torch_type<T>::dtype).device(device()));
+        DeviceMatrixView<T> output_encoding(batch_size, out_w, out_w, reinterpret_cast<T *>(output.data_ptr()));
         std::unique_ptr<Context> model_ctx = encoding_->forward_impl(input_dmv, &output_encoding);
         this->finish();
-        return fromDevice<T>(output_encoding.GetPointer(), {(int64_t)batch_size, (int64_t)out_w});
+        return output;
     }
 
     torch::Tensor inference(const torch::Tensor &input_tensor) override { return forward_pass(input_tensor); }
@@ -170,11 +171,14 @@ template <typename T> class EncodingModule : public Module {
         const uint32_t out_w = encoding_->get_padded_output_width();
         DeviceMatrixView<T> dL_doutput_dmv(batch_size, out_w, out_w, reinterpret_cast<T *>(grad_output.data_ptr()));
         DeviceMatrixView<float> input_encoding_dmv(batch_size, input_width, input_width, input_from_fwd.data_ptr<float>());
-        auto gradients_view = gradients_->GetView();
+        // the scatter overwrites its whole destination: it is the tensor that is handed back; the module keeps a reference
+        // for get_encoding_grads
+        last_gradients_ = torch::empty({(int64_t)encoding_->get_n_params(), 1}, torch::TensorOptions().dtype(torch_type<T>::dtype).device(device()));
+        DeviceMatrixView<T> gradients_view(encoding_->get_n_params(), 1, 1, reinterpret_cast<T *>(last_gradients_.data_ptr()));
         Context ctx;
         encoding_->backward_impl(ctx, input_encoding_dmv, dL_doutput_dmv, &gradients_view);
         this->finish();
-        return {torch::Tensor(), convertDeviceMatrixToTorchTensor(*gradients_)};
+        return {torch::Tensor(), last_gradients_};
     }
 
     torch::Tensor initialize_params() override { return get_params(); }
@@ -206,7 +210,11 @@ template <typename T> class EncodingModule : public Module {
     }
     const void *grid_table() const override { return grid_descriptor() ? encoding_->get_params()->data() : nullptr; }
     std::vector<T> get_encoding_params() { return encoding_->get_params()->copy_to_host(); }
-    std::vector<T> get_encoding_grads() { return gradients_->copy_to_host(); }
+    /// The gradients of the last backward_pass (zeros before the first one).
+    std::vector<T> get_encoding_grads() {
+        if (!last_gradients_.defined()) return std::vector<T>(encoding_->get_n_params(), T(0));
+        return convertTensorToVector<T>(last_gradients_);
+    }
 
   protected:
     void FreeWorkspace() override {
@@ -225,15 +233,10 @@ template <typename T> class EncodingModule : public Module {
     }
 
   private:
-    void initialize_ptr() {
-        if (encoding_ && encoding_->get_n_params()) {
-            gradients_ = std::make_unique<DeviceMatrix<T>>(encoding_->get_n_params(), 1, this->get_queue());
-            gradients_->fill(0.0f).wait();
-        }
-    }
+    void initialize_ptr() {}
 
     std::shared_ptr<Encoding<T>> encoding_;
-    std::unique_ptr<DeviceMatrix<T>> gradients_;
+    torch::Tensor last_gradients_;
     size_t max_batch_size_; // the workspace fits every batch size seen so far
     T *output_encoding_ptr_;
 };

@@ -138,3 +138,49 @@ def test_train_step_with_adam_equals_step_then_update(tnn, dtype, tdt, W, n_hidd
     assert tnn.lib.tnn_mlp_train_step_l2_adam(d, ptr(b["f"]), ptr(b["b"]), ptr(x), ptr(targets), loss_scale, None, None, ptr(b["p"]),
                                               ptr(b["m"]), ptr(b["v"]), 1, *hyper, None, None, M, ptr(ws), 16, None,
                                               tnn.stream()) == _lib.TNN_ERR_WORKSPACE
+
+
+def test_two_streams_give_the_single_stream_results(tnn):
+    """The library keeps no state between calls: calls enqueued on two streams (a network each, its own buffers) give bit
+    for bit what the same calls give one after the other on one stream. Both streams have the default priority."""
+    import ctypes
+
+    from gpu_harness import ptr
+    from tiny_dpcpp_nn import _lib
+
+    gen = torch.Generator(device=tnn.dev).manual_seed(3)
+    cases = []
+    for dtype, tdt, W, n_hidden, M in ((BF16, torch.bfloat16, 64, 4, 1 << 16), (FP16, torch.float16, 32, 2, (1 << 16) + 8)):
+        n_mats = n_hidden + 1
+        desc = tnn.mlp_desc(dtype, W, n_hidden, "relu", "none")
+        master = (torch.rand(n_mats * W * W, device=tnn.dev, generator=gen) * 2 - 1) * (6.0 / (2 * W)) ** 0.5
+        pf, pb = tnn.prepare_packed(desc, master, src_is_fp32=True)
+        x = (torch.rand((M, W), device=tnn.dev, generator=gen) * 2 - 1).to(tdt)
+        g = ((torch.rand((M, W), device=tnn.dev, generator=gen) * 2 - 1) / M).to(tdt)
+        ws_bytes = tnn.lib.tnn_mlp_backward_workspace_bytes(ctypes.byref(desc), M)
+        cases.append(dict(desc=desc, pf=pf, pb=pb, x=x, g=g, M=M, W=W, n_mats=n_mats, tdt=tdt, ws_bytes=ws_bytes))
+
+    def run(case, stream):
+        c, d = case, ctypes.byref(case["desc"])
+        s = ctypes.c_void_p(stream.cuda_stream)
+        out = dict(y=torch.empty_like(c["x"]), interm=torch.empty((c["n_mats"] + 1, c["M"], c["W"]), dtype=c["tdt"], device=tnn.dev),
+                   ib=torch.empty((c["n_mats"], c["M"], c["W"]), dtype=c["tdt"], device=tnn.dev),
+                   dW=torch.empty(c["n_mats"] * c["W"] * c["W"], dtype=torch.float32, device=tnn.dev), dX=torch.empty_like(c["x"]),
+                   ws=torch.empty(c["ws_bytes"], dtype=torch.uint8, device=tnn.dev))
+        for _ in range(3):  # several rounds so that the two streams really overlap
+            _lib.check(tnn.lib.tnn_mlp_inference(d, ptr(c["pf"]), ptr(c["x"]), ptr(out["y"]), c["M"], s))
+            _lib.check(tnn.lib.tnn_mlp_forward(d, ptr(c["pf"]), ptr(c["x"]), ptr(out["interm"]), c["M"], s))
+            _lib.check(tnn.lib.tnn_mlp_backward(d, ptr(c["pb"]), ptr(c["g"]), ptr(out["interm"]), ptr(out["ib"]), ptr(out["dW"]), 1,
+                                                ptr(out["dX"]), c["M"], ptr(out["ws"]), c["ws_bytes"], s))
+        return out
+
+    torch.cuda.synchronize()
+    one = torch.cuda.current_stream()
+    ref = [run(c, one) for c in cases]
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    got = [run(c, st) for c, st in zip(cases, streams)]
+    torch.cuda.synchronize()
+    for r, o in zip(ref, got):
+        for k in ("y", "interm", "ib", "dW", "dX"):
+            assert torch.equal(r[k], o[k]), k

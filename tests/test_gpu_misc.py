@@ -184,3 +184,43 @@ def test_two_streams_give_the_single_stream_results(tnn):
     for r, o in zip(ref, got):
         for k in ("y", "interm", "ib", "dW", "dX"):
             assert torch.equal(r[k], o[k]), k
+
+
+def test_two_host_threads(tnn):
+    """Two host threads, a stream each, call the library at the same time (ctypes releases the GIL during a call): same
+    results as one thread. What the library caches per device lives in thread-local storage."""
+    import ctypes
+    import threading
+
+    from gpu_harness import ptr
+    from tiny_dpcpp_nn import _lib
+
+    gen = torch.Generator(device=tnn.dev).manual_seed(4)
+    W, n_hidden, M = 64, 3, 1 << 15
+    desc = tnn.mlp_desc(BF16, W, n_hidden, "relu", "none")
+    master = (torch.rand((n_hidden + 1) * W * W, device=tnn.dev, generator=gen) * 2 - 1) * 0.2
+    pf, _ = tnn.prepare_packed(desc, master, src_is_fp32=True)
+    xs = [(torch.rand((M, W), device=tnn.dev, generator=gen) * 2 - 1).to(torch.bfloat16) for _ in range(2)]
+    ref = [tnn.inference(desc, pf, x) for x in xs]
+    torch.cuda.synchronize()
+    outs = [torch.empty_like(x) for x in xs]
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    errors = []
+
+    def worker(i):
+        try:
+            s = ctypes.c_void_p(streams[i].cuda_stream)
+            for _ in range(200):
+                _lib.check(tnn.lib.tnn_mlp_inference(ctypes.byref(desc), ptr(pf), ptr(xs[i]), ptr(outs[i]), M, s))
+        except Exception as e:  # noqa: BLE001
+            errors.append(e)
+
+    threads = [threading.Thread(target=worker, args=(i,)) for i in range(2)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    torch.cuda.synchronize()
+    assert not errors, errors
+    for r, o in zip(ref, outs):
+        assert torch.equal(r, o)

@@ -227,6 +227,40 @@ def test_forward_store_routes_at_large_batches(tnn, oracle, dtype, W, n_hidden, 
             assert_propagated(tnn.host(interm_t[l][rows]), ref[l], dtype, f"interm_fwd[{l}] rows {rows}")
 
 
+def test_matrices_beyond_two_gib(tnn, oracle):
+    """A matrix of more than 2 GiB does not fit the 32-bit offsets of the range-checked row stores: forward, inference and
+    backward then take the plain routes. 2^24 + 8 rows of width 64 (2.1 GB per matrix), one hidden layer."""
+    import torch
+    from gpu_harness import TORCH_DT
+    dtype, W, n_hidden, M = BF16, 64, 1, (1 << 24) + 8
+    n_mats = n_hidden + 1
+    w = oracle.round(xavier(W, n_mats, 11), dtype)
+    gen = torch.Generator(device=tnn.dev).manual_seed(12)
+    xt = (torch.rand((M, W), device=tnn.dev, generator=gen) * 2 - 1).to(TORCH_DT[dtype])
+    desc = tnn.mlp_desc(dtype, W, n_hidden, "relu", "none")
+    _, pf, pb = tnn.prepare(desc, w)
+    interm_t = tnn.forward(desc, pf, xt)
+    y_t = tnn.inference(desc, pf, xt)
+    assert torch.equal(interm_t[n_mats], y_t) and torch.equal(interm_t[0], xt)
+    assert not torch.isnan(interm_t[1]).any()
+    gt = ((torch.rand((M, W), device=tnn.dev, generator=gen) * 2 - 1) / M).to(TORCH_DT[dtype])
+    ib, dW, dX = tnn.backward(desc, pb, gt, interm_t, dw_fp32=True)
+    assert not torch.isnan(ib).any() and not torch.isnan(dX).any() and not torch.isnan(dW).any()
+    for rows in (slice(0, 96), slice(M - 96, M)):
+        ref = oracle.mlp_forward_T(dtype, W, n_mats, "relu", "none", w, tnn.host(xt[rows]))
+        for l in range(1, n_mats + 1):
+            assert_propagated(tnn.host(interm_t[l][rows]), ref[l], dtype, f"interm_fwd[{l}] rows {rows}")
+        rib, _, rdX = oracle.mlp_backward_T(dtype, W, n_mats, "relu", "none", w, tnn.host(interm_t[:, rows]), tnn.host(gt[rows]), round_dw=False)
+        for l in range(n_mats):
+            assert_propagated(tnn.host(ib[l][rows]), rib[l], dtype, f"delta[{l}] rows {rows}", scale=1.0 / M)
+        assert_propagated(tnn.host(dX[rows]), rdX, dtype, f"dL/dx rows {rows}", scale=1.0 / M)
+    for l in range(n_mats):
+        exact = torch.zeros((W, W), dtype=torch.float64, device=tnn.dev)
+        for r0 in range(0, M, 1 << 22):  # in pieces: the fp64 copies of whole matrices would take 17 GB each
+            exact += ib[l][r0:r0 + (1 << 22)].double().T @ interm_t[l][r0:r0 + (1 << 22)].double()
+        assert_close(tnn.host(dW[l]), exact.cpu().numpy(), dtype, f"dW[{l}] from the GPU's own deltas")
+
+
 @pytest.mark.parametrize("dtype,W,n_hidden,M", [(BF16, 64, 4, (1 << 18) + 40), (FP16, 32, 2, (1 << 18) + 8), (FP16, 16, 2, (1 << 18) + 24)])
 def test_backward_store_route_at_large_batch(tnn, oracle, dtype, W, n_hidden, M):
     """The fused backward writes its deltas and dL/dx as whole rows from staged tiles, through range-checked buffer stores.

@@ -82,8 +82,7 @@ class _module_function(torch.autograd.Function):
         loss_scale = ctx.loss_scale
 
         if "width" in ctx.info and doutput.shape[1] < ctx.info["width"]:
-            pad = torch.zeros(doutput.shape[0], ctx.info["width"] - doutput.shape[1], device=doutput.device, dtype=doutput.dtype)
-            doutput = torch.hstack((doutput, pad))
+            doutput = torch.nn.functional.pad(doutput, [0, ctx.info["width"] - doutput.shape[1]])  # zeros for the padding columns
 
         batch_size = input.shape[0]
         # loss scaling: 1 for bf16, where the two passes over the gradient (here and after the kernels) are skipped

@@ -20,7 +20,7 @@ import time
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, os.path.join(ROOT, "tiny-dpcpp-nn_amd"))
-sys.path.insert(0, os.path.join(ROOT, "tests"))
+sys.path.insert(0, os.path.join(ROOT, "oracle"))  # the checker (cpu_baseline leg and the parity check only)
 
 PEAK_MFMA_BF16 = 2500.0  # TFLOP/s, dense
 PEAK_HBM = 8000.0  # GB/s
@@ -200,9 +200,9 @@ def main():
     import numpy as np
     import torch
 
-    import gpu_harness
     import oracle_bindings
-    from gpu_harness import ptr
+    from tiny_dpcpp_nn import cabi as gpu_harness
+    from tiny_dpcpp_nn.cabi import ptr
     from tiny_dpcpp_nn import _lib
     from tolerances import BF16, FP16, FP32
 

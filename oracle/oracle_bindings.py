@@ -1,4 +1,5 @@
-"""numpy-in / numpy-out wrappers around oracle/libtnn_oracle.so for the tests."""
+"""numpy-in / numpy-out wrappers around oracle/libtnn_oracle.so: test infrastructure, used by the tests, the smoke check and
+the benchmark's parity check and CPU baseline; never by the product."""
 import ctypes
 from ctypes import c_float, c_int, c_size_t, c_uint32, c_void_p
 

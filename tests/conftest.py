@@ -6,6 +6,7 @@ import pytest
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 sys.path.insert(0, os.path.join(ROOT, "tiny-dpcpp-nn_amd"))
+sys.path.insert(0, os.path.join(ROOT, "oracle"))  # the checker: oracle_bindings, tolerances
 sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
 
 

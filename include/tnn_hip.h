@@ -206,6 +206,22 @@ int tnn_mlp_train_step_l2_adam(const tnn_mlp_desc *desc, void *d_prepared_fwd, v
                                void *d_dLdx, size_t M, void *d_workspace, size_t workspace_bytes, void *main_kernel_done_event,
                                tnn_stream_t stream);
 
+/* tnn_mlp_train_step_l2 for callers that cannot allocate device memory: code recorded into a HIP graph, tight serving
+ * loops, harnesses that forbid hipMalloc. It has no counterpart in the reference. It takes no workspace: the partial
+ * weight gradients and partial losses of the step go to a fixed array of TNN_MLP_TRAIN_STEP_STATIC_SCRATCH_BYTES of
+ * device memory inside the library, which every GPU that runs the library holds until the process ends. The call
+ * allocates and frees nothing. Shapes and batch sizes whose tnn_mlp_train_step_workspace_bytes exceeds that size
+ * (the separate-kernel route of wide or deep networks at large batches) are rejected with TNN_ERR_WORKSPACE; every
+ * shape that has the fused kernel fits at any batch size. Same arguments and results, bit for bit, as
+ * tnn_mlp_train_step_l2. All calls on one GPU share the one array: calls that overlap on a GPU (two streams, two
+ * threads) race; serialise them. Nothing in the array has to be cleared between calls. The first call on a device
+ * looks up the array's address there (make that call outside a graph capture). */
+#define TNN_MLP_TRAIN_STEP_STATIC_SCRATCH_BYTES (21u << 20)
+size_t tnn_mlp_train_step_l2_static_max_bytes(void);
+int tnn_mlp_train_step_l2_static(const tnn_mlp_desc *desc, const void *d_prepared_fwd, const void *d_prepared_bwd,
+                                 const void *d_x, const float *d_targets, float loss_scale, void *d_y, float *d_loss_sum,
+                                 void *d_dW, int dW_is_fp32, void *d_dLdx, size_t M, tnn_stream_t stream);
+
 /* ------------------------------------------------------------------------------------------
  * Multi-resolution hash grid (include/encodings/grid.h, include/common/common_device.h:700-775).
  * ------------------------------------------------------------------------------------------ */

@@ -3,6 +3,8 @@
 #include "adam_update.h"
 #include "tnn_internal.h"
 
+#include <mutex>
+
 namespace tnn {
 
 // loss value summed per workgroup, one atomic per workgroup; gradient rounded to T as in l2.h:24
@@ -131,4 +133,62 @@ TNN_API int tnn_mlp_train_step_l2_adam(const tnn_mlp_desc *desc, void *d_prepare
     if (tail.main_done && hipEventRecord(tail.main_done, s) != hipSuccess) return fail(TNN_ERR_HIP, "hipEventRecord failed");
     return tnn_mlp_adam_update(desc, d_master_packed, d_m, d_v, dW, 1.0f / loss_scale, step, lr, beta1, beta2, eps, d_packed_T,
                                d_prepared_fwd, d_prepared_bwd, stream);
+}
+
+// ------------------------------------------------------------------------------------------------
+// The training step for callers that cannot allocate device memory (code under graph capture, serving loops,
+// harnesses that forbid hipMalloc): the partial weight gradients and partial losses go to a fixed array in
+// device memory that every GPU using this library holds until the process ends.
+// ------------------------------------------------------------------------------------------------
+namespace tnn {
+
+constexpr size_t kStaticScratchBytes = TNN_MLP_TRAIN_STEP_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+// Device address of `scratch` on the current device. In host code the array's name is only a handle for
+// hipGetSymbolAddress; each device has its own copy at its own address, resolved once per device.
+static int static_scratch(void **out) {
+    constexpr int kMaxDevices = 64;
+    static std::mutex mu;
+    static void *addr[kMaxDevices] = {};
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+        (void)hipGetLastError();
+        return fail(TNN_ERR_HIP, "no current HIP device");
+    }
+    std::lock_guard<std::mutex> lock(mu);
+    if (!addr[dev]) {
+        void *p = nullptr;
+        const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p) {
+            (void)hipGetLastError();
+            return fail(TNN_ERR_HIP, "hipGetSymbolAddress(scratch) failed on device %d: %s", dev, hipGetErrorString(e));
+        }
+        addr[dev] = p;
+    }
+    *out = addr[dev];
+    return TNN_OK;
+}
+
+} // namespace tnn
+
+TNN_API size_t tnn_mlp_train_step_l2_static_max_bytes(void) { return kStaticScratchBytes; }
+
+TNN_API int tnn_mlp_train_step_l2_static(const tnn_mlp_desc *desc, const void *d_prepared_fwd, const void *d_prepared_bwd,
+                                         const void *d_x, const float *d_targets, float loss_scale, void *d_y, float *d_loss_sum,
+                                         void *d_dW, int dW_is_fp32, void *d_dLdx, size_t M, tnn_stream_t stream) {
+    int rc = check_mlp_desc(desc);
+    if (rc) return rc;
+    const size_t need = tnn_mlp_train_step_workspace_bytes(desc, M);
+    if (need > kStaticScratchBytes)
+        return fail(TNN_ERR_WORKSPACE,
+                    "this shape and batch size need %zu bytes of scratch memory, the static buffer holds %zu: use "
+                    "tnn_mlp_train_step_l2 with a workspace of the caller's",
+                    need, kStaticScratchBytes);
+    void *ws = nullptr;
+    if ((rc = static_scratch(&ws))) return rc;
+    // Nothing in the buffer has to start at zero: every workgroup overwrites its own partials before the reduction
+    // reads them, and the separate-kernel route writes every matrix before it reads it.
+    return tnn_mlp_train_step_l2(desc, d_prepared_fwd, d_prepared_bwd, d_x, d_targets, loss_scale, d_y, d_loss_sum, d_dW, dW_is_fp32,
+                                 d_dLdx, M, ws, kStaticScratchBytes, stream);
 }

@@ -84,6 +84,12 @@ SIGNATURES = {
         [POINTER(MlpDesc), c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
          c_size_t, c_void_p, c_size_t, c_void_p],
     ),
+    "tnn_mlp_train_step_l2_static_max_bytes": (c_size_t, []),
+    "tnn_mlp_train_step_l2_static": (
+        c_int,
+        [POINTER(MlpDesc), c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
+         c_size_t, c_void_p],
+    ),
     "tnn_adam_step": (
         c_int,
         [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_float, c_size_t, c_int, c_float, c_float, c_float, c_float, c_void_p,

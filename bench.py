@@ -1,29 +1,39 @@
 #!/usr/bin/env python3
-"""Benchmark of the hot path on one MI355X.
+"""Benchmark of the hot path on one MI355X. Prints ONE JSON line.
 
-Default workload (BASELINE config 2, the one the metric is quoted on): one training step of the
-width-64, 4-hidden-layer bf16 fused MLP at batch 2^18 -- forward, L2 loss against U[0,1) targets,
-backward with weight gradients, Adam (lr 1e-3, betas 0.9/0.99, eps 1e-15) on fp32 master weights and
-re-staging of the updated weights for the next step: one tnn_mlp_train_step_l2_adam call, two kernel
-launches. Inputs are resident in HBM before the timed region. Prints ONE JSON line.
+Default run = the whole metric ("fused-MLP train & infer samples/s, w64, batch 2^18"):
+  top level  BASELINE config 2: one training step of the width-64, 4-hidden-layer bf16 fused MLP at batch 2^18 -- forward,
+             L2 loss against U[0,1) targets, backward with weight gradients, Adam (lr 1e-3, betas 0.9/0.99, eps 1e-15) on
+             fp32 master weights and re-staging of the updated weights for the next step: one tnn_mlp_train_step_l2_adam
+             call, two kernel launches
+  "infer"    the same network as fused inference at batch 2^18 (BASELINE config 1's shape at the metric's batch size)
+  "grid"     BASELINE config 5's encoding: 3-D hash grid forward, 2^21 points (the third target of the north star)
+Inputs are resident in HBM before any timed region.
 
-Other workloads (reported as extra lines only when asked for with --workload):
-  infer  BASELINE config 1 shape at batch 2^18: fused inference
-  grid   BASELINE config 5 encoding: 3-D hash grid forward, 2^21 points
+Protocol of every leg: (1) parity of one call against the CPU oracle on the very tensors that are timed (the line carries
+`parity_checked` and the measured differences; a failed check ends the run with an error), (2) `prewarm_ms` of untimed
+calls so that the clocks are up before the declared warm-up, (3) --warmup untimed steps, (4) --reps repetitions (default 5)
+of EXACTLY --steps steps, enqueued back to back on one stream with a HIP event between repetitions and one synchronisation
+at each end; `ms_per_step` is the median repetition and `ms_per_step_reps` lists all of them.
+
+--workload train|infer|grid|train_fb|grid_mlp|grid_train runs one workload on its own (the form the profiles under profiles/
+were collected with); its line has the same top-level fields.
 """
 import argparse
 import ctypes
 import json
 import os
+import statistics
 import sys
 import time
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, os.path.join(ROOT, "tiny-dpcpp-nn_amd"))
-sys.path.insert(0, os.path.join(ROOT, "oracle"))  # the checker (cpu_baseline leg and the parity check only)
+sys.path.insert(0, os.path.join(ROOT, "oracle"))  # the checker: parity check and cpu_baseline leg only
 
 PEAK_MFMA_BF16 = 2500.0  # TFLOP/s, dense
 PEAK_HBM = 8000.0  # GB/s
+METRIC = "fused-MLP train & infer samples/s (w64, batch 2^18); % bf16 MFMA peak"
 
 # HBM-side bytes per launch of each workload's dominant kernel at the default batch sizes, from rocprofv3 counter runs over this
 # file (FETCH_SIZE and WRITE_SIZE, one run each, scaled by what the same counter reads for the --copy-calibration kernel:
@@ -42,30 +52,43 @@ MEASURED_TRAFFIC_BYTES = {
 def parse():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    # a step takes 15-60 us: the first few hundred run while the clocks still ramp up (58.9 us per training step over 200 steps
-    # after 20, 54.0 over 1000 after 200, 53.6 over 2000 after 500), so the defaults time a second of steady state at most
-    ap.add_argument("--steps", type=int, default=1000)
-    ap.add_argument("--warmup", type=int, default=200)
-    ap.add_argument("--workload", default="train", choices=["train", "train_fb", "infer", "grid", "grid_mlp", "grid_train"])
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--reps", type=int, default=5, help="repetitions of --steps timed steps; the median is reported")
+    ap.add_argument("--prewarm-ms", type=float, default=300.0,
+                    help="untimed calls for this long before the declared warm-up (a fresh process starts at idle clocks)")
+    ap.add_argument("--workload", default="all", choices=["all", "train", "train_fb", "infer", "grid", "grid_mlp", "grid_train"])
     ap.add_argument("--batch-log2", type=int, default=None)
     ap.add_argument("--packed-scatter", action="store_true",
                     help="grid_train only: gradient table in fp16 with one packed atomic per feature pair (tnn_grid_backward_packed)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-parity", action="store_true", help="skip the oracle check in front of the timing (profiling runs)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also launch a plain copy kernel (tnn_cast fp32 -> fp32, 256 MiB read + 256 MiB written per launch) so that "
                          "hardware byte counters collected over this run can be scaled by what they read for a known transfer")
     return ap.parse_args()
 
 
+# ------------------------------------------------------------------------------------------------------------------
+# CPU baselines: the oracle (a port of the reference's arithmetic, OpenMP over rows) on a bounded sample
+# ------------------------------------------------------------------------------------------------------------------
+def _timed_loop(fn, budget_s):
+    fn()
+    t0 = time.perf_counter()
+    n = 0
+    while time.perf_counter() - t0 < budget_s:
+        fn()
+        n += 1
+    return n, time.perf_counter() - t0
+
+
 def cpu_baseline_train(oracle, W, n_mats, budget_s=12.0):
-    """The oracle's training step (rounding-point restatement) timed on the host cores on a bounded sample."""
     import numpy as np
     from tolerances import BF16
 
     rng = np.random.default_rng(0)
     lim = np.sqrt(6.0 / (2 * W))
     w = oracle.round(rng.uniform(-lim, lim, (n_mats, W, W)), BF16)
-    cores = oracle.num_threads()
     M = 1 << 14
     x = oracle.round(rng.uniform(-1, 1, (M, W)), BF16)
     tg = rng.uniform(0, 1, (M, W)).astype(np.float32)
@@ -75,14 +98,8 @@ def cpu_baseline_train(oracle, W, n_mats, budget_s=12.0):
         _, g = oracle.l2_loss(BF16, interm[-1], tg, 1.0)
         oracle.mlp_backward_T(BF16, W, n_mats, "relu", "none", w, interm, g, want_dx=False, round_dw=False)
 
-    step()
-    t0 = time.perf_counter()
-    n = 0
-    while time.perf_counter() - t0 < budget_s:
-        step()
-        n += 1
-    dt = time.perf_counter() - t0
-    return {"value": M * n / dt, "unit": "samples/s", "cores": cores, "kind": "port",
+    n, dt = _timed_loop(step, budget_s)
+    return {"value": M * n / dt, "unit": "samples/s", "cores": oracle.num_threads(), "kind": "port",
             "sample": f"{n} training steps (forward, L2, backward with dW) of {M} rows each, w64 / 4 hidden layers, bf16 rounding points, OpenMP over rows"}
 
 
@@ -95,34 +112,28 @@ def cpu_baseline_infer(oracle, W, n_mats, budget_s=12.0):
     w = oracle.round(rng.uniform(-lim, lim, (n_mats, W, W)), BF16)
     M = 1 << 15
     x = oracle.round(rng.uniform(-1, 1, (M, W)), BF16)
-    oracle.mlp_forward_T(BF16, W, n_mats, "relu", "none", w, x, store_interm=False)
-    t0 = time.perf_counter()
-    n = 0
-    while time.perf_counter() - t0 < budget_s:
-        oracle.mlp_forward_T(BF16, W, n_mats, "relu", "none", w, x, store_interm=False)
-        n += 1
-    dt = time.perf_counter() - t0
+    n, dt = _timed_loop(lambda: oracle.mlp_forward_T(BF16, W, n_mats, "relu", "none", w, x, store_interm=False), budget_s)
     return {"value": M * n / dt, "unit": "samples/s", "cores": oracle.num_threads(), "kind": "port",
             "sample": f"{n} inference passes of {M} rows, w64 / 4 hidden layers, bf16 rounding points, OpenMP over rows"}
 
 
-def cpu_baseline_grid(oracle, cfg, budget_s=12.0):
+def _cpu_table(oracle, cfg):
     import numpy as np
     from tolerances import FP16
 
     rng = np.random.default_rng(0)
     off, _, _ = oracle.grid_offsets(cfg["n_dims"], cfg["n_levels"], cfg["log2_hashmap_size"], cfg["base_resolution"], cfg["per_level_scale"])
     n = int(off[-1]) * cfg["n_features_per_level"]
-    table = oracle.round(rng.uniform(-1e-4, 1e-4, n), FP16)
+    return rng, n, oracle.round(rng.uniform(-1e-4, 1e-4, n), FP16)
+
+
+def cpu_baseline_grid(oracle, cfg, budget_s=12.0):
+    import numpy as np
+
+    rng, _, table = _cpu_table(oracle, cfg)
     M = 1 << 16
     x = rng.uniform(0, 1, (M, cfg["n_dims"])).astype(np.float32)
-    oracle.grid_forward(cfg, table, x, 32)
-    t0 = time.perf_counter()
-    k = 0
-    while time.perf_counter() - t0 < budget_s:
-        oracle.grid_forward(cfg, table, x, 32)
-        k += 1
-    dt = time.perf_counter() - t0
+    k, dt = _timed_loop(lambda: oracle.grid_forward(cfg, table, x, 32), budget_s)
     return {"value": M * k / dt, "unit": "points/s", "cores": oracle.num_threads(), "kind": "port",
             "sample": f"{k} forward passes of {M} points through the full 162 MiB table, OpenMP over points"}
 
@@ -131,10 +142,7 @@ def cpu_baseline_grid_mlp(oracle, cfg, w, budget_s=12.0):
     import numpy as np
     from tolerances import FP16
 
-    rng = np.random.default_rng(0)
-    off, _, _ = oracle.grid_offsets(cfg["n_dims"], cfg["n_levels"], cfg["log2_hashmap_size"], cfg["base_resolution"], cfg["per_level_scale"])
-    n = int(off[-1]) * cfg["n_features_per_level"]
-    table = oracle.round(rng.uniform(-1e-4, 1e-4, n), FP16)
+    rng, _, table = _cpu_table(oracle, cfg)
     M = 1 << 16
     x = rng.uniform(0, 1, (M, cfg["n_dims"])).astype(np.float32)
     n_mats = w.shape[0]
@@ -143,13 +151,7 @@ def cpu_baseline_grid_mlp(oracle, cfg, w, budget_s=12.0):
         enc = oracle.round(oracle.grid_forward(cfg, table, x, 64), FP16)
         return oracle.mlp_forward_T(FP16, 64, n_mats, "relu", "none", w, enc, store_interm=False)
 
-    chain()
-    t0 = time.perf_counter()
-    k = 0
-    while time.perf_counter() - t0 < budget_s:
-        chain()
-        k += 1
-    dt = time.perf_counter() - t0
+    k, dt = _timed_loop(chain, budget_s)
     return {"value": M * k / dt, "unit": "points/s", "cores": oracle.num_threads(), "kind": "port",
             "sample": f"{k} passes of {M} points: encoding through the full 162 MiB table, then the 4-matrix network, OpenMP over points"}
 
@@ -160,10 +162,7 @@ def cpu_baseline_grid_train(oracle, cfg, w, budget_s=12.0):
     import numpy as np
     from tolerances import FP16
 
-    rng = np.random.default_rng(0)
-    off, _, _ = oracle.grid_offsets(cfg["n_dims"], cfg["n_levels"], cfg["log2_hashmap_size"], cfg["base_resolution"], cfg["per_level_scale"])
-    n = int(off[-1]) * cfg["n_features_per_level"]
-    table = oracle.round(rng.uniform(-1e-4, 1e-4, n), FP16)
+    rng, n, table = _cpu_table(oracle, cfg)
     M = 1 << 14
     x = rng.uniform(0, 1, (M, cfg["n_dims"])).astype(np.float32)
     targets = np.zeros((M, 64), np.float32)
@@ -177,49 +176,117 @@ def cpu_baseline_grid_train(oracle, cfg, w, budget_s=12.0):
         _, _, d_enc = oracle.mlp_backward_T(FP16, 64, n_mats, "relu", "none", w, interm, grads, round_dw=False)
         oracle.grid_backward(cfg, x, d_enc, n)
 
-    step()
-    t0 = time.perf_counter()
-    k = 0
-    while time.perf_counter() - t0 < budget_s:
-        step()
-        k += 1
-    dt = time.perf_counter() - t0
+    k, dt = _timed_loop(step, budget_s)
     return {"value": M * k / dt, "unit": "samples/s", "cores": oracle.num_threads(), "kind": "port",
             "sample": f"{k} steps of {M} points: encoding, network forward, L2, network backward, scatter into the 7.7 M-entry gradient "
                       "table; OpenMP over points"}
 
 
-def main():
-    args = parse()
-    if args.gpus != 1:
-        print("bench.py measures one GPU: this build has no multi-GPU path. Every batch row is independent, so G GPUs would each take "
-              "M/G rows with a full copy of the weights and exchange the weight gradients once per step; that is not built. "
-              "Run with --gpus 1.", file=sys.stderr)
-        sys.exit(2)
+# ------------------------------------------------------------------------------------------------------------------
+# GPU timing
+# ------------------------------------------------------------------------------------------------------------------
+class Timer:
+    """Pre-warm, warm-up, then `reps` repetitions of exactly `steps` calls, all enqueued back to back on torch's current
+    stream (the stream every launch of this file goes to) with an event between repetitions."""
 
-    import numpy as np
-    import torch
+    def __init__(self, torch, steps, warmup, reps, prewarm_ms):
+        self.torch, self.K, self.W, self.reps, self.prewarm_ms = torch, steps, warmup, reps, prewarm_ms
+        self.n = 0  # calls made so far (the Adam step number follows it)
 
-    import oracle_bindings
-    from tiny_dpcpp_nn import cabi as gpu_harness
-    from tiny_dpcpp_nn.cabi import ptr
-    from tiny_dpcpp_nn import _lib
-    from tolerances import BF16, FP16, FP32
+    def _call(self, fn, k):
+        for _ in range(k):
+            fn(self.n)
+            self.n += 1
 
-    t = gpu_harness.Harness()
-    lib = t.lib
-    oracle = None
-    if not args.no_cpu_baseline:
-        oracle = oracle_bindings.Oracle(os.path.join(ROOT, "oracle", "libtnn_oracle.so"))
+    def run(self, fn, tail=None):
+        """tail: further work enqueued directly behind the last repetition, before the synchronisation (a GPU that idles
+        for a few milliseconds drops its clocks, and the next hundred launches read 10 % slow)."""
+        torch = self.torch
+        t0 = time.perf_counter()
+        while (time.perf_counter() - t0) * 1e3 < self.prewarm_ms:
+            self._call(fn, 50)
+            torch.cuda.synchronize()
+        self._call(fn, self.W)
+        torch.cuda.synchronize()
+        evs = [torch.cuda.Event(enable_timing=True) for _ in range(self.reps + 1)]
+        w0 = time.perf_counter()
+        evs[0].record()
+        for r in range(self.reps):
+            self._call(fn, self.K)
+            evs[r + 1].record()
+        if tail:
+            tail()
+        evs[-1].synchronize()
+        wall = time.perf_counter() - w0
+        torch.cuda.synchronize()
+        per_rep = [evs[r].elapsed_time(evs[r + 1]) / self.K for r in range(self.reps)]
+        return {"ms": statistics.median(per_rep), "reps_ms": per_rep, "wall_ms": wall / (self.K * self.reps) * 1e3}
 
-    K, Wm = args.steps, args.warmup
-    ev = lambda: torch.cuda.Event(enable_timing=True)
-    out = {}
 
-    if args.workload in ("train", "train_fb", "infer"):
+class HipEvents:
+    """Raw HIP events on the launch stream (one the library records between two kernels of a call cannot be a torch event)."""
+
+    def __init__(self):
+        hip = ctypes.CDLL("libamdhip64.so")
+        hip.hipEventCreate.argtypes = [ctypes.POINTER(ctypes.c_void_p)]
+        hip.hipEventRecord.argtypes = [ctypes.c_void_p, ctypes.c_void_p]
+        hip.hipEventElapsedTime.argtypes = [ctypes.POINTER(ctypes.c_float), ctypes.c_void_p, ctypes.c_void_p]
+        self.hip = hip
+
+    def create(self):
+        e = ctypes.c_void_p()
+        assert self.hip.hipEventCreate(ctypes.byref(e)) == 0
+        return e
+
+    def record(self, e, stream):
+        assert self.hip.hipEventRecord(e, stream) == 0
+
+    def elapsed_ms(self, a, b):
+        dt = ctypes.c_float()
+        assert self.hip.hipEventElapsedTime(ctypes.byref(dt), a, b) == 0
+        return dt.value
+
+
+def line(metric, unit, dtype, workload, M, tm, K, Wm, args, roofline, extra=None):
+    out = {"metric": metric, "value": M / (tm["ms"] * 1e-3), "unit": unit, "n_gpus": 1, "steps": K, "warmup": Wm, "ms_per_step": tm["ms"],
+           "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": dtype, "data": "synthetic",
+           "config": {"workload": workload, "batch": M}, "roofline": roofline, "reps": len(tm["reps_ms"]), "ms_per_step_reps": tm["reps_ms"],
+           "prewarm_ms": args.prewarm_ms, "wall_ms_per_step": tm["wall_ms"]}
+    if extra:
+        out.update(extra)
+    return out
+
+
+class Bench:
+    def __init__(self, args):
+        import numpy as np
+        import torch
+
+        from tiny_dpcpp_nn import _lib, cabi
+
+        self.args, self.np, self.torch, self._lib, self.cabi = args, np, torch, _lib, cabi
+        self.t = cabi.Harness()  # raises if the HIP library or the GPU is missing: there is no other path
+        self.lib = self.t.lib
+        self.oracle = None
+        if not (args.no_cpu_baseline and args.no_parity):
+            import oracle_bindings
+            self.oracle = oracle_bindings.Oracle(os.path.join(ROOT, "oracle", "libtnn_oracle.so"))
+        self.K, self.Wm = args.steps, args.warmup
+
+    def timer(self, steps=None, warmup=None):
+        return Timer(self.torch, steps or self.K, warmup if warmup is not None else self.Wm, self.args.reps, self.args.prewarm_ms)
+
+    def check(self, rc):
+        if rc:
+            raise RuntimeError(self.lib.tnn_last_error())
+
+    # --------------------------------------------------------------------------------------------------------------
+    def mlp_case(self):
+        np, torch, t = self.np, self.torch, self.t
+        from tolerances import BF16, FP32
         W, n_hidden = 64, 4
         n_mats = n_hidden + 1
-        M = 1 << (args.batch_log2 or 18)
+        M = 1 << (self.args.batch_log2 or 18)
         desc = t.mlp_desc(BF16, W, n_hidden, "relu", "none")
         rng = np.random.default_rng(42)
         lim = np.sqrt(6.0 / (2 * W))
@@ -229,171 +296,247 @@ def main():
         # fp32 master weights in the packed parameter layout, as the reference's Python module keeps them
         master = t.pack(FP32, W, n_mats, torch.from_numpy(w.reshape(-1)).to(t.dev))
         pf, pb = t.prepare_packed(desc, master, src_is_fp32=True)
+        return dict(W=W, n_hidden=n_hidden, n_mats=n_mats, M=M, desc=desc, w=w, gen=gen, x=x, master=master, pf=pf, pb=pb)
 
-    if args.workload == "train":
-        targets = torch.rand((M, W), device=t.dev, generator=gen)
+    def parity_mlp(self, c, targets):
+        """One training step and one inference on the tensors that are timed, against the oracle. Returns the differences."""
+        np, torch, t, oracle, lib = self.np, self.torch, self.t, self.oracle, self.lib
+        from tiny_dpcpp_nn.cabi import ptr
+        from tolerances import BF16, assert_propagated, max_norm_rel
+        W, n_mats, M, desc = c["W"], c["n_mats"], c["M"], c["desc"]
+        w_T = oracle.round(c["w"], BF16)  # the weights as the kernels see them
+        xh, th = t.host(c["x"]), targets.cpu().numpy()
+        interm = oracle.mlp_forward_T(BF16, W, n_mats, "relu", "none", w_T, xh)
+        res = {}
+        y_inf = t.host(t.inference(desc, c["pf"], c["x"]))
+        assert_propagated(y_inf, interm[-1], BF16, "bench parity: inference output")
+        res["infer_output_max_norm_rel"] = max_norm_rel(y_inf, interm[-1])
+        y, loss, dW, _ = t.train_step_l2(desc, c["pf"], c["pb"], c["x"], targets, 1.0, want_dx=False)
+        yh = t.host(y)
+        assert_propagated(yh, interm[-1], BF16, "bench parity: training-step output")
+        values, grads = oracle.l2_loss(BF16, yh, th, 1.0)
+        ref_loss = float(values.astype(np.float64).sum())
+        assert abs(float(loss.item()) - ref_loss) <= 1e-4 * ref_loss, "bench parity: loss"
+        _, rdW, _ = oracle.mlp_backward_T(BF16, W, n_mats, "relu", "none", w_T, interm, grads, want_dx=False, round_dw=False)
+        dWh = t.host(dW)
+        res["dW_max_norm_rel"] = max(max_norm_rel(dWh[l], rdW[l]) for l in range(n_mats))
+        assert res["dW_max_norm_rel"] < 1e-2, "bench parity: dW"
+        assert_propagated(dWh, rdW, BF16, "bench parity: dW", scale=float(np.abs(rdW).max()))
+        # the timed entry point: the same step with Adam applied in the reduction, on copies of the optimizer state
+        p, m, v = c["master"].clone(), torch.zeros_like(c["master"]), torch.zeros_like(c["master"])
+        pf, pb = c["pf"].clone(), c["pb"].clone()
+        ws_bytes = lib.tnn_mlp_train_step_workspace_bytes(ctypes.byref(desc), M)
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=t.dev)
+        l2 = torch.zeros(1, device=t.dev)
+        self.check(lib.tnn_mlp_train_step_l2_adam(ctypes.byref(desc), ptr(pf), ptr(pb), ptr(c["x"]), ptr(targets), 1.0, None, ptr(l2), ptr(p), ptr(m),
+                                                  ptr(v), 1, 1e-3, 0.9, 0.99, 1e-15, None, None, M, ptr(ws), ws_bytes, None, t.stream()))
+        gp = np.concatenate([oracle.pack_and_transpose(dWh[l].ravel(), W) for l in range(n_mats)])
+        mh = t.host(c["master"])
+        rp, rm, rv = oracle.adam_step(mh, np.zeros_like(mh), np.zeros_like(mh), gp, 1, 1e-3, 0.9, 0.99, 1e-15)
+        assert np.allclose(t.host(p), rp, rtol=1e-6, atol=1e-7) and np.allclose(t.host(m), rm, rtol=1e-6, atol=1e-9), "bench parity: Adam"
+        assert np.allclose(t.host(v), rv, rtol=1e-6, atol=1e-12) and abs(float(l2.item()) - ref_loss) <= 1e-4 * ref_loss, "bench parity: Adam"
+        res["output_max_norm_rel"] = max_norm_rel(yh, interm[-1])
+        res["loss_rel"] = abs(float(loss.item()) - ref_loss) / ref_loss
+        return res
+
+    def leg_train(self, c, targets):
+        np, torch, t, lib = self.np, self.torch, self.t, self.lib
+        from tiny_dpcpp_nn.cabi import ptr
+        W, n_mats, M, desc = c["W"], c["n_mats"], c["M"], c["desc"]
         ws_bytes = lib.tnn_mlp_train_step_workspace_bytes(ctypes.byref(desc), M)
         ws = torch.empty(ws_bytes, dtype=torch.uint8, device=t.dev)
         loss = torch.zeros(1, device=t.dev)
-        m = torch.zeros_like(master)
-        v = torch.zeros_like(master)
-        s = t.stream()
-        d = ctypes.byref(desc)
-        # raw HIP events on the stream the kernels go to: one before the call, one the library records between the
-        # step's main kernel and the reduction + Adam kernel
-        hip = ctypes.CDLL("libamdhip64.so")
-        hip.hipEventCreate.argtypes = [ctypes.POINTER(ctypes.c_void_p)]
-        hip.hipEventRecord.argtypes = [ctypes.c_void_p, ctypes.c_void_p]
-        hip.hipEventElapsedTime.argtypes = [ctypes.POINTER(ctypes.c_float), ctypes.c_void_p, ctypes.c_void_p]
+        master, pf, pb = c["master"], c["pf"], c["pb"]
+        m, v = torch.zeros_like(master), torch.zeros_like(master)
+        s, d = t.stream(), ctypes.byref(desc)
+        a = (ptr(pf), ptr(pb), ptr(c["x"]), ptr(targets), ptr(loss), ptr(master), ptr(m), ptr(v), ptr(ws))
+        hip = HipEvents()
 
-        def hip_event():
-            e = ctypes.c_void_p()
-            assert hip.hipEventCreate(ctypes.byref(e)) == 0
-            return e
-
-        ks, ke = [hip_event() for _ in range(K)], [hip_event() for _ in range(K)]
-
-        def step(i, timed=-1):
-            mid = None
-            if timed >= 0:
-                assert hip.hipEventRecord(ks[timed], s) == 0
-                mid = ke[timed]
-            rc = lib.tnn_mlp_train_step_l2_adam(d, ptr(pf), ptr(pb), ptr(x), ptr(targets), 1.0, None, ptr(loss), ptr(master), ptr(m), ptr(v),
-                                                i + 1, 1e-3, 0.9, 0.99, 1e-15, None, None, M, ptr(ws), ws_bytes, mid, s)
+        def step(i, mid=None):
+            rc = lib.tnn_mlp_train_step_l2_adam(d, a[0], a[1], a[2], a[3], 1.0, None, a[4], a[5], a[6], a[7], i + 1, 1e-3, 0.9, 0.99, 1e-15,
+                                                None, None, M, a[8], ws_bytes, mid, s)
             if rc:
                 raise RuntimeError(lib.tnn_last_error())
 
-        for i in range(Wm):
-            step(i)
+        step(0)
         torch.cuda.synchronize()
         loss0 = float(loss.item())
-        e0, e1 = ev(), ev()
-        t0 = time.perf_counter()
-        e0.record()
-        for i in range(K):
-            step(Wm + i)
-        e1.record()
-        torch.cuda.synchronize()
-        wall = time.perf_counter() - t0
-        ms = e0.elapsed_time(e1) / K
-        # a second pass of K steps, each bracketed by HIP events on the launch stream, for the kernel's own duration
-        # (kept out of the timed region above: an event between two launches costs about a microsecond)
-        for i in range(K):
-            step(Wm + K + i, timed=i)
-        torch.cuda.synchronize()
-        kern_ms = 0.0
-        for a, b in zip(ks, ke):
-            dt = ctypes.c_float()
-            assert hip.hipEventElapsedTime(ctypes.byref(dt), a, b) == 0
-            kern_ms += dt.value / K
-        flops = 3 * 2 * M * W * W * n_mats  # reference convention: forward + backward-data + dW
-        out = {
-            "metric": "fused-MLP train & infer samples/s (w64, batch 2^18); % bf16 MFMA peak",
-            "value": M / (ms * 1e-3), "unit": "samples/s", "n_gpus": 1, "steps": K, "warmup": Wm, "ms_per_step": ms,
-            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
-            "config": {"workload": f"training step: w64, 4 hidden layers (5 matmuls), ReLU/linear, bf16, batch 2^{int(np.log2(M))}, "
-                                   "L2 loss, Adam on fp32 masters (BASELINE config 2)", "batch": M},
-            "roofline": {"bound": "mfma", "achieved": flops / (kern_ms * 1e-3) / 1e12, "peak": PEAK_MFMA_BF16, "unit": "TFLOP/s",
-                         "frac": flops / (kern_ms * 1e-3) / 1e12 / PEAK_MFMA_BF16,
-                         "traffic": MEASURED_TRAFFIC_BYTES.get(("train", int(np.log2(M)))),
-                         "kernel": "mlp_train_fused_kernel (forward + loss + backward + partial dW)", "kernel_ms": kern_ms,
-                         "algorithmic_flops_per_launch": flops},
-            "mfma_frac_whole_step": flops / (ms * 1e-3) / 1e12 / PEAK_MFMA_BF16,
-            "wall_ms_per_step": wall / K * 1e3,
-            "loss_first": loss0, "loss_last": float(loss.item()),
-        }
-        if oracle is not None:
-            out["cpu_baseline"] = cpu_baseline_train(oracle, W, n_mats)
+        timer = self.timer()
+        timer.n = 1
+        # behind the timed repetitions, a further pass with each step bracketed by HIP events on the launch stream (one
+        # recorded here in front of the call, one the library records between the main kernel and the reduction), for the
+        # main kernel's own duration; kept out of the timed region: the two events cost about 6 us per step
+        nk = 50
+        ks, ke = [hip.create() for _ in range(nk)], [hip.create() for _ in range(nk)]
 
-    elif args.workload == "train_fb":
+        def bracketed():
+            for i in range(nk):
+                hip.record(ks[i], s)
+                step(timer.n + i, ke[i])
+
+        tm = timer.run(step, tail=bracketed)
+        kern_ms = statistics.median(hip.elapsed_ms(x, y) for x, y in zip(ks, ke))
+        flops = 3 * 2 * M * W * W * n_mats  # reference convention: forward + backward-data + dW
+        lg = int(np.log2(M))
+        ach = flops / (kern_ms * 1e-3) / 1e12
+        roof = {"bound": "mfma", "achieved": ach, "peak": PEAK_MFMA_BF16, "unit": "TFLOP/s", "frac": ach / PEAK_MFMA_BF16,
+                "traffic": MEASURED_TRAFFIC_BYTES.get(("train", lg)), "kernel": "mlp_train_fused_kernel (forward + loss + backward + partial dW)",
+                "kernel_ms": kern_ms, "algorithmic_flops_per_launch": flops}
+        return line(METRIC, "samples/s", "bf16",
+                    f"training step: w64, 4 hidden layers (5 matmuls), ReLU/linear, bf16, batch 2^{lg}, L2 loss, Adam on fp32 masters (BASELINE config 2)",
+                    M, tm, self.K, self.Wm, self.args, roof,
+                    {"mfma_frac_whole_step": flops / (tm["ms"] * 1e-3) / 1e12 / PEAK_MFMA_BF16, "loss_first": loss0, "loss_last": float(loss.item())})
+
+    def leg_infer(self, c):
+        np, torch, t, lib = self.np, self.torch, self.t, self.lib
+        from tiny_dpcpp_nn.cabi import ptr
+        W, n_mats, M, desc = c["W"], c["n_mats"], c["M"], c["desc"]
+        y = torch.empty_like(c["x"])
+        s, d = t.stream(), ctypes.byref(desc)
+        a = (ptr(c["pf"]), ptr(c["x"]), ptr(y))
+
+        def step(i):
+            if lib.tnn_mlp_inference(d, a[0], a[1], a[2], M, s):
+                raise RuntimeError(lib.tnn_last_error())
+
+        tm = self.timer().run(step)
+        flops = 2 * M * W * W * n_mats
+        bytes_ = 2 * M * W * 2 + n_mats * W * W * 2
+        lg = int(np.log2(M))
+        ach = bytes_ / (tm["ms"] * 1e-3) / 1e9
+        roof = {"bound": "hbm", "achieved": ach, "peak": PEAK_HBM, "unit": "GB/s", "frac": ach / PEAK_HBM,
+                "traffic": MEASURED_TRAFFIC_BYTES.get(("infer", lg)), "kernel": "mlp_forward_kernel (inference)", "kernel_ms": tm["ms"],
+                "algorithmic_bytes_per_launch": bytes_, "mfma_frac": flops / (tm["ms"] * 1e-3) / 1e12 / PEAK_MFMA_BF16}
+        return line(METRIC, "samples/s", "bf16",
+                    f"inference: w64, 4 hidden layers (5 matmuls), ReLU/linear, bf16, batch 2^{lg} (BASELINE config 1 shape)",
+                    M, tm, self.K, self.Wm, self.args, roof, {"mfma_frac": roof["mfma_frac"]})
+
+    # --------------------------------------------------------------------------------------------------------------
+    def grid_case(self):
+        torch, t = self.torch, self.t
+        from tolerances import FP16
+        cfg = dict(n_dims=3, n_levels=16, n_features_per_level=2, log2_hashmap_size=22, base_resolution=16, per_level_scale=1.447)
+        M = 1 << (self.args.batch_log2 or 21)
+        gd = t.grid_desc(cfg, FP16)
+        n = t.grid_n_params(gd)
+        gen = torch.Generator(device=t.dev).manual_seed(7)
+        table = (torch.rand(n, device=t.dev, generator=gen) * 2e-4 - 1e-4).to(torch.float16)
+        x = torch.rand((M, 3), device=t.dev, generator=gen)
+        return dict(cfg=cfg, M=M, gd=gd, n=n, table=table, x=x)
+
+    def parity_grid(self, g, out_rows, width, what, mlp=None):
+        """The first 2^14 points of the timed batch through the oracle: cell selection bit-exact, values within the fp16 bar."""
+        np, t, oracle = self.np, self.t, self.oracle
+        from tolerances import FP16, assert_close, assert_propagated, max_norm_rel
+        n = min(g["M"], 1 << 14)
+        xs = g["x"][:n].contiguous()
+        assert np.array_equal(t.grid_indices(g["gd"], xs), oracle.grid_indices(g["cfg"], xs.cpu().numpy())), "bench parity: grid indices"
+        table = t.host(g["table"])
+        if mlp is None:
+            ref = oracle.grid_forward(g["cfg"], table, xs.cpu().numpy(), width)
+            assert_close(t.host(out_rows[:n]), ref, FP16, what, scale=1e-4)
+            return {"grid_indices": "bit-exact", "grid_values_max_norm_rel": max_norm_rel(t.host(out_rows[:n]), ref)}
+        enc = oracle.round(oracle.grid_forward(g["cfg"], table, xs.cpu().numpy(), 64), FP16)
+        ref = oracle.mlp_forward_T(FP16, 64, mlp.shape[0], "relu", "none", mlp, enc, store_interm=False)
+        assert_propagated(t.host(out_rows[:n]), ref, FP16, what, scale=float(np.abs(ref).max()))
+        return {"grid_indices": "bit-exact", "output_max_norm_rel": max_norm_rel(t.host(out_rows[:n]), ref)}
+
+    def leg_grid(self, g, fused_mlp=False):
+        np, torch, t, lib = self.np, self.torch, self.t, self.lib
+        from tiny_dpcpp_nn.cabi import ptr
+        from tolerances import FP16
+        M, gd = g["M"], g["gd"]
+        s = t.stream()
+        K, Wm = min(self.K, 50), min(self.Wm, 5)
+        w = None
+        if not fused_mlp:
+            o = torch.empty((M, 32), dtype=torch.float16, device=t.dev)
+            a = (ctypes.byref(gd), ptr(g["x"]), ptr(g["table"]), ptr(o))
+            call = lambda i: lib.tnn_grid_forward(a[0], a[1], a[2], a[3], FP16, 32, M, s)
+            bpp = 12 + 16 * 8 * 4 + 32 * 2
+        else:
+            # BASELINE config 5 whole: the encoding feeds a width-64 network with 3 hidden layers (16 real outputs) in one kernel
+            W, n_hidden, n_out = 64, 3, 16
+            mdesc = t.mlp_desc(FP16, W, n_hidden, "relu", "none")
+            rng = np.random.default_rng(42)
+            lim = np.sqrt(6.0 / (2 * W))
+            w = rng.uniform(-lim, lim, (n_hidden + 1, W, W)).astype(np.float32)
+            w[0, 32:, :] = 0
+            w[-1, :, n_out:] = 0
+            _, pf, _ = t.prepare(mdesc, w)
+            o = torch.empty((M, W), dtype=torch.float16, device=t.dev)
+            a = (ctypes.byref(gd), ctypes.byref(mdesc), ptr(g["x"]), ptr(g["table"]), ptr(pf), ptr(o))
+            call = lambda i: lib.tnn_grid_mlp_inference(a[0], a[1], a[2], a[3], a[4], a[5], M, s)
+            bpp = 12 + 16 * 8 * 4 + W * 2  # coordinates + gathers + the padded output row; the encoded row stays on chip
+        self.check(call(0))
+        torch.cuda.synchronize()
+        parity = None
+        if self.oracle is not None and not self.args.no_parity:
+            parity = self.parity_grid(g, o, 32, "bench parity: encoding", mlp=self.oracle.round(w, FP16) if fused_mlp else None)
+        tm = self.timer(K, Wm).run(call)
+        lg = int(np.log2(M))
+        ach = bpp * M / (tm["ms"] * 1e-3) / 1e9
+        name = "grid_mlp" if fused_mlp else "grid"
+        roof = {"bound": "hbm", "achieved": ach, "peak": PEAK_HBM, "unit": "GB/s", "frac": ach / PEAK_HBM,
+                "traffic": MEASURED_TRAFFIC_BYTES.get((name, lg)), "kernel": "grid_mlp_inference_kernel" if fused_mlp else "grid_forward_kernel",
+                "kernel_ms": tm["ms"], "algorithmic_bytes_per_launch": bpp * M}
+        out = line("hash-grid + fused-MLP inference points/s (3-D, 16x2, log2 22, fp16; w64, 3 hidden layers; batch 2^21); % HBM peak" if fused_mlp else
+                   "hash-grid forward points/s (3-D, 16x2, log2 22, fp16 table, batch 2^21); % HBM peak", "points/s", "f16",
+                   (f"3-D hash-grid encoding + w64/3-hidden-layer network inference in one kernel, 2^{lg} points (BASELINE config 5)" if fused_mlp else
+                    f"3-D hash-grid encoding forward, 2^{lg} points (BASELINE config 5 encoding)"), M, tm, K, Wm, self.args, roof,
+                   {"parity_checked": parity is not None, "parity": parity})
+        return out, w
+
+    # --------------------------------------------------------------------------------------------------------------
+    def leg_train_fb(self, c):
         # The reference's own training step (Trainer::training_step, include/trainer.h:23-46): a forward pass that stores every
         # activation, then a backward pass that returns the weight gradients, the deltas and dL/dx. No loss, no optimizer.
-        d = ctypes.byref(desc)
-        s = t.stream()
-        g = (torch.rand((M, W), device=t.dev, generator=gen) * 2 - 1).to(torch.bfloat16) / M
+        np, torch, t, lib, _lib = self.np, self.torch, self.t, self.lib, self._lib
+        from tiny_dpcpp_nn.cabi import ptr
+        W, n_mats, M, desc = c["W"], c["n_mats"], c["M"], c["desc"]
+        d, s = ctypes.byref(desc), t.stream()
+        g = (torch.rand((M, W), device=t.dev, generator=c["gen"]) * 2 - 1).to(torch.bfloat16) / M
         interm_f = torch.empty((n_mats + 1, M, W), dtype=torch.bfloat16, device=t.dev)
         interm_b = torch.empty((n_mats, M, W), dtype=torch.bfloat16, device=t.dev)
         dW = torch.empty(n_mats * W * W, dtype=torch.bfloat16, device=t.dev)
-        dX = torch.empty_like(x)
+        dX = torch.empty_like(c["x"])
         ws_bytes = lib.tnn_mlp_backward_workspace_bytes(d, M)
         ws = torch.empty(ws_bytes, dtype=torch.uint8, device=t.dev)
-        mid = ev()
+        mid, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
 
-        def step(timed=False):
-            _lib.check(lib.tnn_mlp_forward(d, ptr(pf), ptr(x), ptr(interm_f), M, s))
+        def step(i, timed=False):
+            _lib.check(lib.tnn_mlp_forward(d, ptr(c["pf"]), ptr(c["x"]), ptr(interm_f), M, s))
             if timed:
                 mid.record()
-            _lib.check(lib.tnn_mlp_backward(d, ptr(pb), ptr(g), ptr(interm_f), ptr(interm_b), ptr(dW), 0, ptr(dX), M, ptr(ws), ws_bytes, s))
+            _lib.check(lib.tnn_mlp_backward(d, ptr(c["pb"]), ptr(g), ptr(interm_f), ptr(interm_b), ptr(dW), 0, ptr(dX), M, ptr(ws), ws_bytes, s))
 
-        for _ in range(Wm):
-            step()
-        torch.cuda.synchronize()
-        e0, e1 = ev(), ev()
-        e0.record()
-        for _ in range(K):
-            step()
-        e1.record()
-        torch.cuda.synchronize()
-        ms = e0.elapsed_time(e1) / K
-        bwd_ms = 0.0
+        tm = self.timer().run(step)
+        bwd = []
         for _ in range(10):  # the backward call on its own, outside the timed region
-            step(timed=True)
-            e1.record()
+            step(0, timed=True)
+            end.record()
             torch.cuda.synchronize()
-            bwd_ms += mid.elapsed_time(e1) / 10
+            bwd.append(mid.elapsed_time(end))
+        bwd_ms = statistics.median(bwd)
         flops = 3 * 2 * M * W * W * n_mats
-        # bytes of the backward call: dL/dy and n_mats activation matrices in, n_mats delta matrices and dL/dx out
-        bwd_bytes = (2 * n_mats + 2) * M * W * 2
-        out = {
-            "metric": "fused-MLP train & infer samples/s (w64, batch 2^18); % bf16 MFMA peak",
-            "value": M / (ms * 1e-3), "unit": "samples/s", "n_gpus": 1, "steps": K, "warmup": Wm, "ms_per_step": ms,
-            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
-            "config": {"workload": f"training step as the reference's Trainer runs it: forward_pass with stored activations + backward_pass "
-                                   f"(deltas, dW, dL/dx), w64, 4 hidden layers, bf16, batch 2^{int(np.log2(M))}; no loss, no optimizer", "batch": M},
-            "roofline": {"bound": "hbm", "achieved": bwd_bytes / (bwd_ms * 1e-3) / 1e9, "peak": PEAK_HBM, "unit": "GB/s",
-                         "frac": bwd_bytes / (bwd_ms * 1e-3) / 1e9 / PEAK_HBM, "traffic": MEASURED_TRAFFIC_BYTES.get(("train_fb", int(np.log2(M)))),
-                         "kernel": "mlp_backward_fused_kernel (+ train_reduce_kernel)", "kernel_ms": bwd_ms,
-                         "algorithmic_bytes_per_launch": bwd_bytes},
-            "mfma_frac_whole_step": flops / (ms * 1e-3) / 1e12 / PEAK_MFMA_BF16,
-        }
-        if oracle is not None:
-            out["cpu_baseline"] = cpu_baseline_train(oracle, W, n_mats)
+        bwd_bytes = (2 * n_mats + 2) * M * W * 2  # dL/dy and n_mats activation matrices in, n_mats delta matrices and dL/dx out
+        lg = int(np.log2(M))
+        ach = bwd_bytes / (bwd_ms * 1e-3) / 1e9
+        roof = {"bound": "hbm", "achieved": ach, "peak": PEAK_HBM, "unit": "GB/s", "frac": ach / PEAK_HBM,
+                "traffic": MEASURED_TRAFFIC_BYTES.get(("train_fb", lg)), "kernel": "mlp_backward_fused_kernel (+ train_reduce_kernel)",
+                "kernel_ms": bwd_ms, "algorithmic_bytes_per_launch": bwd_bytes}
+        return line(METRIC, "samples/s", "bf16",
+                    f"training step as the reference's Trainer runs it: forward_pass with stored activations + backward_pass (deltas, dW, dL/dx), "
+                    f"w64, 4 hidden layers, bf16, batch 2^{lg}; no loss, no optimizer", M, tm, self.K, self.Wm, self.args, roof,
+                    {"mfma_frac_whole_step": flops / (tm["ms"] * 1e-3) / 1e12 / PEAK_MFMA_BF16})
 
-    elif args.workload == "infer":
-        y = torch.empty_like(x)
-        s = t.stream()
-        d = ctypes.byref(desc)
-        for _ in range(Wm):
-            lib.tnn_mlp_inference(d, ptr(pf), ptr(x), ptr(y), M, s)
-        torch.cuda.synchronize()
-        e0, e1 = ev(), ev()
-        e0.record()
-        for _ in range(K):
-            lib.tnn_mlp_inference(d, ptr(pf), ptr(x), ptr(y), M, s)
-        e1.record()
-        torch.cuda.synchronize()
-        ms = e0.elapsed_time(e1) / K
-        flops = 2 * M * W * W * n_mats
-        bytes_ = 2 * M * W * 2 + n_mats * W * W * 2
-        out = {
-            "metric": "fused-MLP train & infer samples/s (w64, batch 2^18); % bf16 MFMA peak",
-            "value": M / (ms * 1e-3), "unit": "samples/s", "n_gpus": 1, "steps": K, "warmup": Wm, "ms_per_step": ms,
-            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
-            "config": {"workload": f"inference: w64, 4 hidden layers (5 matmuls), ReLU/linear, bf16, batch 2^{int(np.log2(M))} (BASELINE config 1 shape)",
-                       "batch": M},
-            "roofline": {"bound": "hbm", "achieved": bytes_ / (ms * 1e-3) / 1e9, "peak": PEAK_HBM, "unit": "GB/s",
-                         "frac": bytes_ / (ms * 1e-3) / 1e9 / PEAK_HBM, "traffic": MEASURED_TRAFFIC_BYTES.get(("infer", int(np.log2(M)))),
-                         "kernel": "mlp_forward_kernel (inference)",
-                         "kernel_ms": ms, "algorithmic_bytes_per_launch": bytes_},
-            "mfma_frac": flops / (ms * 1e-3) / 1e12 / PEAK_MFMA_BF16,
-        }
-        if oracle is not None:
-            out["cpu_baseline"] = cpu_baseline_infer(oracle, W, n_mats)
-
-    elif args.workload == "grid_train":
+    def leg_grid_train(self):
         # BASELINE config 4: 2-D hash grid -> w64 network with 2 hidden layers, 3 real outputs, one whole optimisation step:
         # encoding, fused network step (forward, L2, backward, dL/d(encoding), Adam on the weights), scatter into the gradient
         # table, Adam on the table's fp32 master with the fp16 table re-rounded
+        np, torch, t, lib, _lib, args = self.np, self.torch, self.t, self.lib, self._lib, self.args
+        from tiny_dpcpp_nn.cabi import ptr
+        from tolerances import FP16, FP32
         cfg = dict(n_dims=2, n_levels=16, n_features_per_level=2, log2_hashmap_size=19, base_resolution=16, per_level_scale=1.5)
         W, n_hidden, n_out = 64, 2, 3
         M = 1 << (args.batch_log2 or 18)
@@ -428,7 +571,7 @@ def main():
         s = t.stream()
         g = ctypes.byref(gd)
         hyper = (1e-3, 0.9, 0.99, 1e-15)
-        k0, k1 = ev(), ev()
+        k0, k1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
 
         def step(i, time_scatter=False):
             _lib.check(lib.tnn_grid_forward(g, ptr(x), ptr(table), ptr(enc), FP16, W, M, s))
@@ -445,106 +588,108 @@ def main():
             _lib.check(lib.tnn_adam_step(ptr(table_master), ptr(mt), ptr(vt), ptr(grad_table), FP16 if args.packed_scatter else FP32,
                                          1.0 / loss_scale, n, i + 1, *hyper, ptr(table), FP16, s))
 
-        K = min(K, 50)
-        Wm = min(Wm, 5)
-        for i in range(Wm):
-            step(i)
+        K, Wm = min(self.K, 50), min(self.Wm, 5)
+        step(0)
         torch.cuda.synchronize()
         loss0 = float(loss.item()) * W / n_out  # mean over the real outputs
-        e0, e1 = ev(), ev()
-        e0.record()
-        for i in range(K):
-            step(Wm + i)
-        e1.record()
-        torch.cuda.synchronize()
-        ms = e0.elapsed_time(e1) / K
-        scatter_ms = 0.0
+        timer = self.timer(K, Wm)
+        timer.n = 1
+        tm = timer.run(step)
+        sc = []
         for i in range(10):  # the scatter (fill of the gradient table + atomics) on its own, outside the timed region
-            step(Wm + K + i, time_scatter=True)
+            step(timer.n + i, time_scatter=True)
             torch.cuda.synchronize()
-            scatter_ms += k0.elapsed_time(k1) / 10
+            sc.append(k0.elapsed_time(k1))
+        scatter_ms = statistics.median(sc)
         # algorithmic bytes of the scatter per point: coordinates + dL/d(encoding) row + read-modify-write of 16 levels x 4 corners x
         # 2 features (4-byte gradients: 1096 B; 2-byte: 584 B)
         gb = 2 if args.packed_scatter else 4
         bpp = 8 + 32 * 2 + 16 * 4 * 2 * gb * 2
-        out = {
-            "metric": "hash-grid + fused-MLP training samples/s (2-D, 16x2, log2 19; w64, 2 hidden layers; batch 2^18; whole step with both Adam updates)",
-            "value": M / (ms * 1e-3), "unit": "samples/s", "n_gpus": 1, "steps": K, "warmup": Wm, "ms_per_step": ms,
-            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
-            "config": {"workload": f"2-D hash-grid encoding + w64/2-hidden-layer network, one optimisation step, 2^{int(np.log2(M))} points "
-                                   f"(BASELINE config 4; gradient table {'fp16, packed atomics' if args.packed_scatter else 'fp32'})", "batch": M},
-            "roofline": {"bound": "hbm", "achieved": bpp * M / (scatter_ms * 1e-3) / 1e9, "peak": PEAK_HBM, "unit": "GB/s",
-                         "frac": bpp * M / (scatter_ms * 1e-3) / 1e9 / PEAK_HBM,
-                         "traffic": MEASURED_TRAFFIC_BYTES.get(("grid_train_packed" if args.packed_scatter else "grid_train", int(np.log2(M)))),
-                         "kernel": "grid_backward_kernel (with the fill of the gradient table in front of it)",
-                         "kernel_ms": scatter_ms, "algorithmic_bytes_per_launch": bpp * M},
-            "loss_first": loss0, "loss_last": float(loss.item()) * W / n_out,
-        }
-        if oracle is not None:
+        lg = int(np.log2(M))
+        ach = bpp * M / (scatter_ms * 1e-3) / 1e9
+        roof = {"bound": "hbm", "achieved": ach, "peak": PEAK_HBM, "unit": "GB/s", "frac": ach / PEAK_HBM,
+                "traffic": MEASURED_TRAFFIC_BYTES.get(("grid_train_packed" if args.packed_scatter else "grid_train", lg)),
+                "kernel": "grid_backward_kernel (with the fill of the gradient table in front of it)", "kernel_ms": scatter_ms,
+                "algorithmic_bytes_per_launch": bpp * M}
+        out = line("hash-grid + fused-MLP training samples/s (2-D, 16x2, log2 19; w64, 2 hidden layers; batch 2^18; whole step with both Adam updates)",
+                   "samples/s", "f16",
+                   f"2-D hash-grid encoding + w64/2-hidden-layer network, one optimisation step, 2^{lg} points "
+                   f"(BASELINE config 4; gradient table {'fp16, packed atomics' if args.packed_scatter else 'fp32'})", M, tm, K, Wm, args, roof,
+                   {"loss_first": loss0, "loss_last": float(loss.item()) * W / n_out})
+        return out, cfg, w
+
+
+def sub(leg):
+    """A leg as a sub-object of the default line: the fields that differ from the top level."""
+    keep = ("value", "unit", "ms_per_step", "ms_per_step_reps", "steps", "warmup", "dtype", "config", "roofline", "mfma_frac", "parity_checked",
+            "parity", "cpu_baseline")
+    return {k: leg[k] for k in keep if k in leg}
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path. Every batch row is independent, so G GPUs would each take "
+              "M/G rows with a full copy of the weights and exchange the weight gradients once per step; that is not built. "
+              "Run with --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+
+    b = Bench(args)
+    torch, oracle = b.torch, b.oracle
+    from tolerances import FP16
+    do_parity = oracle is not None and not args.no_parity
+    do_cpu = oracle is not None and not args.no_cpu_baseline
+    wl = args.workload
+
+    if wl in ("all", "train", "infer", "train_fb"):
+        c = b.mlp_case()
+        targets = torch.rand((c["M"], c["W"]), device=b.t.dev, generator=c["gen"])
+        parity = b.parity_mlp(c, targets) if (do_parity and wl != "train_fb") else None
+    if wl in ("all", "train"):
+        out = b.leg_train(c, targets)
+        out.update({"parity_checked": parity is not None, "parity": parity})
+        if do_cpu:
+            out["cpu_baseline"] = cpu_baseline_train(oracle, c["W"], c["n_mats"])
+    if wl in ("all", "infer"):
+        # the training leg has moved the weights; inference is timed on whatever they are now (its parity ran on the initial ones)
+        inf = b.leg_infer(c)
+        inf.update({"parity_checked": parity is not None, "parity": parity})
+        if do_cpu:
+            inf["cpu_baseline"] = cpu_baseline_infer(oracle, c["W"], c["n_mats"], budget_s=6.0 if wl == "all" else 12.0)
+        if wl == "all":
+            out["infer"] = sub(inf)
+        else:
+            out = inf
+    if wl == "train_fb":
+        out = b.leg_train_fb(c)
+        if do_cpu:
+            out["cpu_baseline"] = cpu_baseline_train(oracle, c["W"], c["n_mats"])
+    if wl in ("all", "grid", "grid_mlp"):
+        if wl == "all":
+            del c, targets
+            torch.cuda.empty_cache()
+        g = b.grid_case()
+        leg, w = b.leg_grid(g, fused_mlp=(wl == "grid_mlp"))
+        if do_cpu:
+            leg["cpu_baseline"] = (cpu_baseline_grid_mlp(oracle, g["cfg"], oracle.round(w, FP16)) if wl == "grid_mlp" else
+                                   cpu_baseline_grid(oracle, g["cfg"], budget_s=6.0 if wl == "all" else 12.0))
+        if wl == "all":
+            out["grid"] = sub(leg)
+        else:
+            out = leg
+    if wl == "grid_train":
+        out, cfg, w = b.leg_grid_train()
+        if do_cpu:
             out["cpu_baseline"] = cpu_baseline_grid_train(oracle, cfg, oracle.round(w, FP16))
 
-    else:
-        cfg = dict(n_dims=3, n_levels=16, n_features_per_level=2, log2_hashmap_size=22, base_resolution=16, per_level_scale=1.447)
-        M = 1 << (args.batch_log2 or 21)
-        gd = t.grid_desc(cfg, FP16)
-        n = t.grid_n_params(gd)
-        gen = torch.Generator(device=t.dev).manual_seed(7)
-        table = (torch.rand(n, device=t.dev, generator=gen) * 2e-4 - 1e-4).to(torch.float16)
-        x = torch.rand((M, 3), device=t.dev, generator=gen)
-        s = t.stream()
-        K = min(K, 50)
-        if args.workload == "grid":
-            o = torch.empty((M, 32), dtype=torch.float16, device=t.dev)
-            call = lambda: lib.tnn_grid_forward(ctypes.byref(gd), ptr(x), ptr(table), ptr(o), FP16, 32, M, s)
-            bpp = 12 + 16 * 8 * 4 + 32 * 2
-        else:
-            # BASELINE config 5 whole: the encoding feeds a width-64 network with 3 hidden layers (16 real outputs) in one kernel
-            W, n_hidden, n_out = 64, 3, 16
-            mdesc = t.mlp_desc(FP16, W, n_hidden, "relu", "none")
-            rng = np.random.default_rng(42)
-            lim = np.sqrt(6.0 / (2 * W))
-            w = rng.uniform(-lim, lim, (n_hidden + 1, W, W)).astype(np.float32)
-            w[0, 32:, :] = 0
-            w[-1, :, n_out:] = 0
-            _, pf, _ = t.prepare(mdesc, w)
-            o = torch.empty((M, W), dtype=torch.float16, device=t.dev)
-            call = lambda: lib.tnn_grid_mlp_inference(ctypes.byref(gd), ctypes.byref(mdesc), ptr(x), ptr(table), ptr(pf), ptr(o), M, s)
-            bpp = 12 + 16 * 8 * 4 + W * 2  # coordinates + gathers + the padded output row; the encoded row stays on chip
-        for _ in range(min(Wm, 5)):
-            rc = call()
-            if rc:
-                raise RuntimeError(lib.tnn_last_error())
-        torch.cuda.synchronize()
-        e0, e1 = ev(), ev()
-        e0.record()
-        for _ in range(K):
-            call()
-        e1.record()
-        torch.cuda.synchronize()
-        ms = e0.elapsed_time(e1) / K
-        grid_only = args.workload == "grid"
-        out = {
-            "metric": ("hash-grid forward points/s (3-D, 16x2, log2 22, fp16 table, batch 2^21); % HBM peak" if grid_only else
-                       "hash-grid + fused-MLP inference points/s (3-D, 16x2, log2 22, fp16; w64, 3 hidden layers; batch 2^21); % HBM peak"),
-            "value": M / (ms * 1e-3), "unit": "points/s", "n_gpus": 1, "steps": K, "warmup": min(Wm, 5), "ms_per_step": ms,
-            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
-            "config": {"workload": (f"3-D hash-grid encoding forward, 2^{int(np.log2(M))} points (BASELINE config 5 encoding)" if grid_only else
-                                    f"3-D hash-grid encoding + w64/3-hidden-layer network inference in one kernel, 2^{int(np.log2(M))} points "
-                                    "(BASELINE config 5)"), "batch": M},
-            "roofline": {"bound": "hbm", "achieved": bpp * M / (ms * 1e-3) / 1e9, "peak": PEAK_HBM, "unit": "GB/s",
-                         "frac": bpp * M / (ms * 1e-3) / 1e9 / PEAK_HBM, "traffic": MEASURED_TRAFFIC_BYTES.get((args.workload, int(np.log2(M)))),
-                         "kernel": "grid_forward_kernel" if grid_only else "grid_mlp_inference_kernel",
-                         "kernel_ms": ms, "algorithmic_bytes_per_launch": bpp * M},
-        }
-        if oracle is not None:
-            out["cpu_baseline"] = cpu_baseline_grid(oracle, cfg) if grid_only else cpu_baseline_grid_mlp(oracle, cfg, oracle.round(w, FP16))
-
     if args.copy_calibration:
+        from tiny_dpcpp_nn.cabi import ptr
+        from tolerances import FP32
         n = 64 << 20
-        src = torch.ones(n, dtype=torch.float32, device=t.dev)
+        src = torch.ones(n, dtype=torch.float32, device=b.t.dev)
         dst = torch.empty_like(src)
         for _ in range(3):
-            _lib.check(lib.tnn_cast(FP32, ptr(dst), FP32, ptr(src), n, t.stream()))
+            b._lib.check(b.lib.tnn_cast(FP32, ptr(dst), FP32, ptr(src), n, b.t.stream()))
         torch.cuda.synchronize()
 
     print(json.dumps(out))

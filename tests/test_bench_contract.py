@@ -21,10 +21,18 @@ def test_more_than_one_gpu_is_refused_with_a_message():
     assert "one GPU" in r.stderr and r.stdout.strip() == ""
 
 
+def check_roofline(roof):
+    for key in ROOFLINE:
+        assert key in roof, key
+    assert abs(roof["frac"] - roof["achieved"] / roof["peak"]) < 1e-9
+    assert roof["bound"] in ("hbm", "mfma") and roof["unit"] in ("GB/s", "TFLOP/s")
+
+
 @pytest.mark.gpu
-@pytest.mark.parametrize("workload", ["train", "train_fb", "infer", "grid", "grid_mlp", "grid_train"])
-def test_every_workload_prints_the_contract_line(workload):
-    r = subprocess.run([sys.executable, BENCH, "--workload", workload, "--steps", "5", "--warmup", "2", "--no-cpu-baseline"],
+def test_default_run_carries_the_whole_metric():
+    """No --workload: the training step at the top level, inference and the 3-D encoding as sub-objects, each checked against
+    the oracle before it is timed, each the median of the repetitions."""
+    r = subprocess.run([sys.executable, BENCH, "--steps", "5", "--warmup", "2", "--reps", "3", "--prewarm-ms", "20", "--no-cpu-baseline"],
                        capture_output=True, text=True, timeout=600)
     assert r.returncode == 0, r.stderr[-2000:]
     lines = [l for l in r.stdout.splitlines() if l.strip()]
@@ -32,9 +40,29 @@ def test_every_workload_prints_the_contract_line(workload):
     out = json.loads(lines[0])
     for key in REQUIRED:
         assert key in out, key
-    for key in ROOFLINE:
-        assert key in out["roofline"], key
+    assert out["steps"] == 5 and out["warmup"] == 2 and out["reps"] == 3 and len(out["ms_per_step_reps"]) == 3
+    assert sorted(out["ms_per_step_reps"])[1] == out["ms_per_step"]
+    assert out["parity_checked"] is True and out["parity"]["dW_max_norm_rel"] < 1e-2
+    check_roofline(out["roofline"])
+    assert out["roofline"]["bound"] == "mfma" and "training step" in out["config"]["workload"]
+    for leg, unit in (("infer", "samples/s"), ("grid", "points/s")):
+        assert out[leg]["unit"] == unit and out[leg]["value"] > 0 and out[leg]["parity_checked"] is True
+        check_roofline(out[leg]["roofline"])
+        assert out[leg]["roofline"]["bound"] == "hbm"
+    assert 0 < out["infer"]["roofline"]["mfma_frac"] < 1
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("workload", ["train", "train_fb", "infer", "grid", "grid_mlp", "grid_train"])
+def test_every_workload_prints_the_contract_line(workload):
+    r = subprocess.run([sys.executable, BENCH, "--workload", workload, "--steps", "5", "--warmup", "2", "--reps", "2", "--prewarm-ms", "20",
+                        "--no-cpu-baseline"], capture_output=True, text=True, timeout=600)
+    assert r.returncode == 0, r.stderr[-2000:]
+    lines = [l for l in r.stdout.splitlines() if l.strip()]
+    assert len(lines) == 1
+    out = json.loads(lines[0])
+    for key in REQUIRED:
+        assert key in out, key
+    check_roofline(out["roofline"])
     assert out["n_gpus"] == 1 and out["vs_baseline"] is None and out["data"] == "synthetic"
     assert "workload" in out["config"] and out["value"] > 0
-    assert abs(out["roofline"]["frac"] - out["roofline"]["achieved"] / out["roofline"]["peak"]) < 1e-9
-    assert out["roofline"]["bound"] in ("hbm", "mfma") and out["roofline"]["unit"] in ("GB/s", "TFLOP/s")

@@ -206,6 +206,14 @@ int tnn_mlp_train_step_l2_adam(const tnn_mlp_desc *desc, void *d_prepared_fwd, v
                                void *d_dLdx, size_t M, void *d_workspace, size_t workspace_bytes, void *main_kernel_done_event,
                                tnn_stream_t stream);
 
+/* Testing aid, no counterpart in the reference. In the width-64 training and backward kernels the four waves that share
+ * staged tiles meet at a counter in LDS; a wave waits there for at most `iterations` polls (default 2^22, far beyond any
+ * real wait) so that a kernel always ends. A wave whose wait runs out marks its workgroup, and the call then delivers NaN
+ * in the loss and in EVERY weight gradient (and, through Adam, in the weights) instead of a plausible wrong number.
+ * Setting the limit to 0 forces that path from the host while every kernel still runs to its end. Returns the previous
+ * limit; process-wide. */
+int tnn_debug_set_meeting_spin_limit(int iterations);
+
 /* tnn_mlp_train_step_l2 for callers that cannot allocate device memory: code recorded into a HIP graph, tight serving
  * loops, harnesses that forbid hipMalloc. It has no counterpart in the reference. It takes no workspace: the partial
  * weight gradients and partial losses of the step go to a fixed array of TNN_MLP_TRAIN_STEP_STATIC_SCRATCH_BYTES of

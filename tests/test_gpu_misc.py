@@ -224,3 +224,43 @@ def test_two_host_threads(tnn):
     assert not errors, errors
     for r, o in zip(ref, outs):
         assert torch.equal(r, o)
+
+
+def test_a_meeting_that_gives_up_poisons_the_step(tnn, oracle):
+    """The waves of the width-64 training kernels meet at an LDS counter with a bounded wait. With the bound forced to 0
+    from the host every wait gives up at once; every kernel still runs to its end, and the call must then return NaN in
+    the loss and in every weight gradient, never a plausible number. Back at the default bound the same call is right."""
+    import torch
+    from gpu_harness import ptr
+    from tiny_dpcpp_nn import _lib
+    dtype, W, n_hidden, M = BF16, 64, 4, 1 << 17  # two rounds per wave: the first has meetings
+    n_mats = n_hidden + 1
+    rng = np.random.default_rng(5)
+    lim = np.sqrt(6.0 / (2 * W))
+    w = oracle.round(rng.uniform(-lim, lim, (n_mats, W, W)), dtype)
+    x = oracle.round(rng.uniform(-1, 1, (M, W)), dtype)
+    desc = tnn.mlp_desc(dtype, W, n_hidden, "relu", "none")
+    _, pf, pb = tnn.prepare(desc, w)
+    xt = tnn.dev_tensor(x, dtype)
+    tt = torch.from_numpy(rng.uniform(0, 1, (M, W)).astype(np.float32)).to(tnn.dev)
+    good = tnn.train_step_l2(desc, pf, pb, xt, tt, 1.0)
+    torch.cuda.synchronize()
+    old = tnn.lib.tnn_debug_set_meeting_spin_limit(0)
+    try:
+        assert old == 1 << 22
+        y, loss, dW, dX = tnn.train_step_l2(desc, pf, pb, xt, tt, 1.0)
+        interm = tnn.forward(desc, pf, xt)
+        g = (torch.rand((M, W), device=tnn.dev) / M).to(torch.bfloat16)
+        _, dW_b, dX_b = tnn.backward(desc, pb, g, interm, dw_fp32=True)
+        torch.cuda.synchronize()
+    finally:
+        assert tnn.lib.tnn_debug_set_meeting_spin_limit(old) == 0
+    assert torch.isnan(loss).all() and torch.isnan(dW).all(), "a step whose waits gave up must not return numbers"
+    assert torch.isnan(dW_b).all()
+    # what does not depend on other waves' tiles is still right
+    assert torch.equal(y.view(torch.int16), good[0].view(torch.int16)) and torch.equal(dX.view(torch.int16), good[3].view(torch.int16))
+    again = tnn.train_step_l2(desc, pf, pb, xt, tt, 1.0)
+    torch.cuda.synchronize()
+    for a, b in zip(again, good):
+        assert torch.equal(a.view(torch.uint8), b.view(torch.uint8))
+    assert tnn.lib.tnn_debug_set_meeting_spin_limit(-1) == _lib.TNN_ERR_INVALID_ARGUMENT

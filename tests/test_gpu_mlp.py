@@ -347,6 +347,31 @@ def test_baseline_config_2_training_step(tnn, oracle):
     assert np.allclose(tnn.host(p), rp, rtol=1e-6, atol=1e-7)
     assert np.allclose(tnn.host(m), rm, rtol=1e-6, atol=1e-9) and np.allclose(tnn.host(v), rv, rtol=1e-6, atol=1e-12)
     assert np.array_equal(tnn.host(pT), oracle.round(tnn.host(p), BF16))
+    # the one-call entry point (the one the benchmark times): same step with Adam applied inside the gradient reduction
+    p2 = torch.from_numpy(master.copy()).to(tnn.dev)
+    m2, v2 = torch.zeros_like(p2), torch.zeros_like(p2)
+    pT2 = torch.empty(p2.shape, dtype=torch.bfloat16, device=tnn.dev)
+    pf2, pb2 = pf.clone(), pb.clone()
+    y2, dX2 = torch.empty_like(xt), torch.empty_like(xt)
+    loss2 = torch.full((1,), float("nan"), device=tnn.dev)
+    ws_bytes = tnn.lib.tnn_mlp_train_step_workspace_bytes(ctypes.byref(desc), M)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=tnn.dev)
+    _lib.check(tnn.lib.tnn_mlp_train_step_l2_adam(ctypes.byref(desc), ptr(pf2), ptr(pb2), ptr(xt), ptr(tt), 1.0, ptr(y2), ptr(loss2), ptr(p2),
+                                                  ptr(m2), ptr(v2), 1, 1e-3, 0.9, 0.99, 1e-15, ptr(pT2), ptr(dX2), M, ptr(ws), ws_bytes, None,
+                                                  tnn.stream()))
+    assert_propagated(tnn.host(y2), interm[-1], dtype, "output of the one-call step")
+    assert abs(float(loss2.item()) - float(values.astype(np.float64).sum())) < 1e-4 * float(values.astype(np.float64).sum())
+    # dL/dx: bit-equal to the step without Adam; against the oracle's backward over the oracle's own forward the elementwise
+    # bar holds, while single rows whose ReLU mask flipped on a rounding boundary are outside any max-norm bound
+    assert torch.equal(dX2.view(torch.int16), dX.view(torch.int16))
+    from tolerances import PROPAGATED
+    assert_close(tnn.host(dX2), rdX, dtype, "dL/dx of the one-call step", scale=1.0 / M, frac_ok=PROPAGATED)
+    assert np.allclose(tnn.host(p2), rp, rtol=1e-6, atol=1e-7)
+    assert np.allclose(tnn.host(m2), rm, rtol=1e-6, atol=1e-9) and np.allclose(tnn.host(v2), rv, rtol=1e-6, atol=1e-12)
+    assert np.array_equal(tnn.host(pT2), oracle.round(tnn.host(p2), BF16))
+    # the weights it re-staged for the next step are the rounded masters in both operand orders
+    wf_ref, wb_ref = tnn.prepare_packed(desc, p2, src_is_fp32=True)
+    assert torch.equal(pf2.view(torch.int16), wf_ref.view(torch.int16)) and torch.equal(pb2.view(torch.int16), wb_ref.view(torch.int16))
 
 
 def test_linearity_property_full_size(tnn, oracle):

@@ -1,7 +1,12 @@
 // Launch plan and dispatch of the fused training step (kernels: mlp_train.inc, compiled per storage type).
 #include "mlp_train_shape.h"
 
+#include <atomic>
+
 namespace tnn {
+
+static std::atomic<int> g_meeting_spin_limit{1 << 22};
+int meeting_spin_limit() { return g_meeting_spin_limit.load(std::memory_order_relaxed); }
 
 static constexpr size_t kMaxLds = 160 * 1024;
 
@@ -71,3 +76,8 @@ size_t fused_train_workspace_bytes(const tnn_mlp_desc *d, size_t M) {
 }
 
 } // namespace tnn
+
+TNN_API int tnn_debug_set_meeting_spin_limit(int iterations) {
+    if (iterations < 0) return tnn::fail(TNN_ERR_INVALID_ARGUMENT, "the spin limit cannot be negative");
+    return tnn::g_meeting_spin_limit.exchange(iterations, std::memory_order_relaxed);
+}

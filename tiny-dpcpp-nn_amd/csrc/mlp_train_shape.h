@@ -32,6 +32,9 @@ struct FusedPlan {
 
 FusedPlan fused_plan(const tnn_mlp_desc *d, size_t M);
 
+// Iterations a wave waits at a meeting of the waves that share staged tiles before it gives up (tnn_debug_set_meeting_spin_limit).
+int meeting_spin_limit();
+
 // per storage type (mlp_train_bf16.hip / mlp_train_fp16.hip)
 int fused_train_launch_bf16(const tnn_mlp_desc *d, const FusedPlan &p, const void *wf, const void *wb, const void *x,
                             const float *targets, float loss_scale, void *y, float *loss_sum, void *dW, int dW_is_fp32, void *dx,

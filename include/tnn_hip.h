@@ -277,6 +277,20 @@ size_t tnn_grid_n_params(const tnn_grid_desc *desc);
 int tnn_grid_forward(const tnn_grid_desc *desc, const float *d_x, const void *d_table, void *d_out, int out_dtype,
                      uint32_t padded_width, size_t M, tnn_stream_t stream);
 
+/* Cell order of a batch, for large batches of scattered points. No counterpart in the reference, whose kernel_grid takes the
+ * points as they come (include/encodings/grid.h:37-135, launch :696-731). tnn_grid_order_points writes, into a caller-owned
+ * buffer of tnn_grid_order_bytes(desc, M) bytes (256-byte aligned), one 16-byte record per point, coordinates and row number,
+ * sorted by the cell of a coarse grid (counting sort on the leading 6 bits of every coordinate in 3-D, 9 in 2-D; coordinates
+ * outside [0, 1) and NaN land in an end bin). tnn_grid_forward_ordered is tnn_grid_forward reading those records: thread i
+ * evaluates the i-th record and writes that point's row, so d_out equals tnn_grid_forward's bit for bit, while neighbouring
+ * lanes gather from the same 128-byte lines of the table (config 5, 2^21 uniform points: 1.8 ms -> 1.0 ms + the ordering).
+ * The records depend on d_x only: one ordering serves any number of forward calls on the same points. M < 2^32. */
+size_t tnn_grid_order_bytes(const tnn_grid_desc *desc, size_t M);
+int tnn_grid_order_points(const tnn_grid_desc *desc, const float *d_x, size_t M, void *d_order, size_t order_bytes,
+                          tnn_stream_t stream);
+int tnn_grid_forward_ordered(const tnn_grid_desc *desc, const void *d_order, const void *d_table, void *d_out, int out_dtype,
+                             uint32_t padded_width, size_t M, tnn_stream_t stream);
+
 /* kernel_grid_backward with GradientMode::Overwrite or Accumulate (include/encodings/grid.h:137-245,
  * 736-797). d_dLdy: M x padded_width of dy_dtype. d_grad_table: n_params fp32 (grad_t = float,
  * grid.h:586). overwrite != 0 zeroes the table first (grid.h:758-762). */

@@ -1,0 +1,117 @@
+"""Cell order of a batch (tnn_grid_order_points) and the forward pass that reads it (tnn_grid_forward_ordered): the records are
+a permutation of the rows with their own coordinates, sorted by coarse cell, and the encoded rows equal tnn_grid_forward's bit
+for bit whatever the distribution of the points."""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+from tolerances import FP16, FP32, assert_close
+
+pytestmark = pytest.mark.gpu
+
+CFG4 = dict(n_dims=2, n_levels=16, n_features_per_level=2, log2_hashmap_size=19, base_resolution=16, per_level_scale=1.5)
+CFG5 = dict(n_dims=3, n_levels=16, n_features_per_level=2, log2_hashmap_size=22, base_resolution=16, per_level_scale=1.447)
+
+
+def points(kind, M, D, rng):
+    if kind == "uniform":
+        return rng.uniform(0, 1, (M, D)).astype(np.float32)
+    if kind == "clustered":  # nearly everything in one coarse bin: the refinement's long-bin path
+        x = (0.3 + 0.01 * rng.uniform(0, 1, (M, D))).astype(np.float32)
+        x[::97] = rng.uniform(0, 1, (len(x[::97]), D))
+        return x
+    if kind == "identical":
+        return np.full((M, D), 0.625, np.float32)
+    x = rng.uniform(-0.5, 1.5, (M, D)).astype(np.float32)  # outside the unit cube, infinities and NaN among them
+    x[3 % M], x[5 % M], x[7 % M] = np.nan, np.inf, -np.inf
+    x[11 % M, 0] = np.nan
+    return x
+
+
+def records_of(tnn, d, xt):
+    M = xt.shape[0]
+    buf = tnn.grid_order(d, xt)
+    torch.cuda.synchronize()
+    rec = buf[: M * 16].view(torch.float32).reshape(M, 4).cpu().numpy()
+    return buf, rec, rec[:, 3].copy().view(np.uint32)
+
+
+@pytest.mark.parametrize("cfg", [CFG4, CFG5])
+@pytest.mark.parametrize("kind", ["uniform", "clustered", "identical", "wild"])
+@pytest.mark.parametrize("M", [1, 8, 1000, 4096 + 24, 300000])
+def test_order_is_a_permutation_and_forward_is_unchanged(tnn, cfg, kind, M):
+    D = cfg["n_dims"]
+    rng = np.random.default_rng(M + D)
+    x = points(kind, M, D, rng)
+    xt = torch.from_numpy(x).to(tnn.dev)
+    d = tnn.grid_desc(cfg, FP16)
+    buf, rec, rows = records_of(tnn, d, xt)
+    assert np.array_equal(np.sort(rows), np.arange(M, dtype=np.uint32)), "every row exactly once"
+    assert np.array_equal(rec[:, :D].view(np.uint32), x[rows].view(np.uint32)), "a record carries its own row's coordinates"
+    # sorted by the coarse key: the leading bits of every coordinate, first dimension fastest
+    bits = 4 if D == 3 else 6
+    with np.errstate(invalid="ignore", over="ignore"):
+        s = x[rows].astype(np.float32) * np.float32(1 << bits)
+        q = np.where(s > 0, np.minimum(np.where(np.isfinite(s), s, np.float32(1 << bits)), (1 << bits) - 1), 0).astype(np.int64)
+    key = sum(q[:, k] << (bits * k) for k in range(D))
+    assert np.all(np.diff(key) >= 0), "records are not in coarse-cell order"
+    n = tnn.grid_n_params(d)
+    table = torch.from_numpy(rng.uniform(-1, 1, n).astype(np.float32)).to(tnn.dev).to(torch.float16)
+    if kind == "wild":
+        xt = torch.nan_to_num(xt, nan=0.25, posinf=1.5, neginf=-0.5)  # the encoding of a NaN coordinate is not defined
+        buf = tnn.grid_order(d, xt)
+    plain = tnn.grid_forward(d, xt, table, 48, FP16)
+    ordered = tnn.grid_forward_ordered(d, buf, table, 48, M, FP16)
+    torch.cuda.synchronize()
+    assert torch.equal(plain.view(torch.int16), ordered.view(torch.int16))
+
+
+def test_ordered_forward_matches_the_oracle_and_every_variant(tnn, oracle):
+    rng = np.random.default_rng(3)
+    for cfg, pd, od in ((dict(CFG5, n_features_per_level=4, n_levels=8, interpolation="Smoothstep"), FP32, FP32),
+                        (dict(CFG4, grid_type="Dense", n_levels=6, n_features_per_level=1), FP16, FP16),
+                        (dict(CFG5, hash="Prime", n_features_per_level=8, n_levels=4, interpolation="Nearest"), FP16, FP32)):
+        M = 20000
+        x = rng.uniform(0, 1, (M, cfg["n_dims"])).astype(np.float32)
+        d = tnn.grid_desc(cfg, pd)
+        n = tnn.grid_n_params(d)
+        table = oracle.round(rng.uniform(-1, 1, n), pd)
+        tt = torch.from_numpy(table).to(tnn.dev).to(torch.float16 if pd == FP16 else torch.float32)
+        xt = torch.from_numpy(x).to(tnn.dev)
+        width = cfg["n_levels"] * cfg["n_features_per_level"]
+        out = tnn.grid_forward_ordered(d, tnn.grid_order(d, xt), tt, width, M, od)
+        ref = oracle.grid_forward(cfg, table, x, width)
+        assert_close(out.to(torch.float32).cpu().numpy(), ref, od, f"ordered forward {cfg}")
+        assert torch.equal(out.view(torch.uint8), tnn.grid_forward(d, xt, tt, width, od).view(torch.uint8))
+
+
+def test_order_buffer_checks(tnn):
+    from tiny_dpcpp_nn import _lib
+    d = tnn.grid_desc(CFG5, FP16)
+    x = torch.rand((64, 3), device=tnn.dev)
+    need = tnn.lib.tnn_grid_order_bytes(ctypes.byref(d), 64)
+    assert need >= 64 * 16
+    buf = torch.empty(need + 256, dtype=torch.uint8, device=tnn.dev)
+    p = buf.data_ptr()
+    assert tnn.lib.tnn_grid_order_points(ctypes.byref(d), x.data_ptr(), 64, p, need - 1, None) == _lib.TNN_ERR_WORKSPACE
+    assert tnn.lib.tnn_grid_order_points(ctypes.byref(d), x.data_ptr(), 64, p + 16, need, None) == _lib.TNN_ERR_INVALID_ARGUMENT
+    assert tnn.lib.tnn_grid_order_points(ctypes.byref(d), x.data_ptr(), 0, p, need, None) == _lib.TNN_ERR_INVALID_ARGUMENT
+    assert tnn.lib.tnn_grid_order_bytes(ctypes.byref(d), 0) == 0
+
+
+def test_config_5_full_size_ordered(tnn, oracle):
+    """BASELINE config 5's encoding at 2^21 points in cell order: equal to the plain pass bit for bit, a sample against the oracle."""
+    M = 1 << 21
+    d = tnn.grid_desc(CFG5, FP16)
+    n = tnn.grid_n_params(d)
+    gen = torch.Generator(device=tnn.dev).manual_seed(5)
+    table = (torch.rand(n, device=tnn.dev, generator=gen) * 2e-4 - 1e-4).to(torch.float16)
+    x = torch.rand((M, 3), device=tnn.dev, generator=gen)
+    plain = tnn.grid_forward(d, x, table, 32, FP16)
+    ordered = tnn.grid_forward_ordered(d, tnn.grid_order(d, x), table, 32, M, FP16)
+    assert torch.equal(plain.view(torch.int16), ordered.view(torch.int16))
+    rows = torch.randint(0, M, (4096,), device=tnn.dev, generator=gen)
+    ref = oracle.grid_forward(CFG5, table.float().cpu().numpy(), x[rows].cpu().numpy(), 32)
+    assert_close(ordered[rows].float().cpu().numpy(), ref, FP16, "config 5 ordered", scale=1e-4)

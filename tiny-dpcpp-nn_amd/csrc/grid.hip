@@ -45,30 +45,46 @@ constexpr int kGridThreads = 256;
 // 16-byte pieces (a per-level 4-byte store turns into a 32-byte masked write at the memory controller).
 template <int D, int F, typename P, typename O>
 __global__ void __launch_bounds__(kGridThreads)
-    grid_forward_kernel(const GridLevels lv, const GridParams gp, const float *__restrict__ xin, const P *__restrict__ table,
-                        O *__restrict__ out, long long M) {
+    grid_forward_kernel(const GridLevels lv, const GridParams gp, const float *__restrict__ xin, const float4 *__restrict__ order,
+                        const P *__restrict__ table, O *__restrict__ out, long long M) {
     constexpr int PER16 = 16 / (int)sizeof(O);            // outputs per 16-byte piece
     constexpr int GL = (PER16 / F) > 0 ? (PER16 / F) : 1; // levels per group (F = 8 with fp32 output: 1 level, 2 pieces)
     constexpr int NOUT = GL * F;
     typedef O ovec __attribute__((ext_vector_type(NOUT)));
     const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= M) return;
+    // In cell order (grid_order.hip) thread i takes the i-th record, coordinates and row number, instead of row i.
     float x[D];
+    long long row = i;
+    if (order) {
+        const float4 r = order[i];
+        x[0] = r.x;
+        x[1] = r.y;
+        if (D > 2) x[D - 1] = r.z;
+        row = (long long)__float_as_uint(r.w);
+    } else {
 #pragma unroll
-    for (int d = 0; d < D; ++d) x[d] = xin[i * D + d];
-    O *orow = out + i * gp.padded_width;
+        for (int d = 0; d < D; ++d) x[d] = xin[i * D + d];
+    }
+    O *orow = out + row * gp.padded_width;
     const bool row_aligned = ((gp.padded_width * sizeof(O)) % 16 == 0) && ((reinterpret_cast<uintptr_t>(out) & 15) == 0);
 
-    for (uint32_t l0 = 0; l0 < gp.n_levels; l0 += GL) {
+    // The first kHeld pieces of a row (128 bytes with 16-byte pieces) are kept in registers and stored together when the
+    // last of them is done, so that a row's pieces reach L2 back to back and leave it as one write; pieces computed
+    // thousands of cycles apart would each sit in L2 as a partly written line among the table's lines.
+    constexpr int kHeld = (NOUT * sizeof(O) == 16) ? 8 : 0;
+    ovec held[kHeld > 0 ? kHeld : 1];
+    auto do_group = [&](const uint32_t l0, ovec &o) __attribute__((always_inline)) {
         LevelConst lc[GL];
 #pragma unroll
         for (int gl = 0; gl < GL; ++gl) lc[gl] = level_const(lv, (l0 + gl < gp.n_levels) ? l0 + gl : l0);
         const int n_valid = (int)((gp.n_levels - l0 < (uint32_t)GL) ? gp.n_levels - l0 : (uint32_t)GL);
         float r[NOUT];
         encode_levels<D, F, P, GL>(lc, n_valid, gp, x, table, r);
-        ovec o;
 #pragma unroll
         for (int e = 0; e < NOUT; ++e) o[e] = to_out<O>(r[e]);
+    };
+    auto store_group = [&](const uint32_t l0, const ovec &o) __attribute__((always_inline)) {
         const uint32_t col0 = l0 * F;
         if (row_aligned && l0 + GL <= gp.n_levels) {
             if constexpr (NOUT * sizeof(O) == 16) {
@@ -82,6 +98,17 @@ __global__ void __launch_bounds__(kGridThreads)
             for (int e = 0; e < NOUT; ++e)
                 if (l0 + e / F < gp.n_levels) orow[col0 + e] = o[e];
         }
+    };
+#pragma unroll
+    for (int p = 0; p < kHeld; ++p)
+        if ((uint32_t)(p * GL) < gp.n_levels) do_group((uint32_t)(p * GL), held[p]);
+#pragma unroll
+    for (int p = 0; p < kHeld; ++p)
+        if ((uint32_t)(p * GL) < gp.n_levels) store_group((uint32_t)(p * GL), held[p]);
+    for (uint32_t l0 = kHeld * GL; l0 < gp.n_levels; l0 += GL) {
+        ovec o;
+        do_group(l0, o);
+        store_group(l0, o);
     }
     // zero padding of the row (include/encodings/grid.h:682-694), in 16-byte pieces where the row allows it
     uint32_t c = gp.n_levels * F;
@@ -297,20 +324,20 @@ int check_grid_desc(const tnn_grid_desc *d) {
 }
 
 template <int D, int F, typename P>
-static int launch_grid_forward_o(const GridLevels &lv, const GridParams &gp, const float *x, const void *table, void *out,
-                                 int out_dtype, size_t M, hipStream_t s) {
+static int launch_grid_forward_o(const GridLevels &lv, const GridParams &gp, const float *x, const float4 *order, const void *table,
+                                 void *out, int out_dtype, size_t M, hipStream_t s) {
     const unsigned blocks = (unsigned)((M + kGridThreads - 1) / kGridThreads);
     switch (out_dtype) {
     case TNN_FP32:
-        TNN_LAUNCH((grid_forward_kernel<D, F, P, float>), dim3(blocks), dim3(kGridThreads), 0, s, lv, gp, x, (const P *)table,
+        TNN_LAUNCH((grid_forward_kernel<D, F, P, float>), dim3(blocks), dim3(kGridThreads), 0, s, lv, gp, x, order, (const P *)table,
                            (float *)out, (long long)M);
         break;
     case TNN_BF16:
-        TNN_LAUNCH((grid_forward_kernel<D, F, P, bf16_t>), dim3(blocks), dim3(kGridThreads), 0, s, lv, gp, x, (const P *)table,
+        TNN_LAUNCH((grid_forward_kernel<D, F, P, bf16_t>), dim3(blocks), dim3(kGridThreads), 0, s, lv, gp, x, order, (const P *)table,
                            (bf16_t *)out, (long long)M);
         break;
     case TNN_FP16:
-        TNN_LAUNCH((grid_forward_kernel<D, F, P, fp16_t>), dim3(blocks), dim3(kGridThreads), 0, s, lv, gp, x, (const P *)table,
+        TNN_LAUNCH((grid_forward_kernel<D, F, P, fp16_t>), dim3(blocks), dim3(kGridThreads), 0, s, lv, gp, x, order, (const P *)table,
                            (fp16_t *)out, (long long)M);
         break;
     default: return fail(TNN_ERR_UNSUPPORTED, "out_dtype %d", out_dtype);
@@ -319,10 +346,10 @@ static int launch_grid_forward_o(const GridLevels &lv, const GridParams &gp, con
 }
 
 template <int D, int F>
-static int launch_grid_forward_p(const tnn_grid_desc *d, const GridLevels &lv, const GridParams &gp, const float *x,
+static int launch_grid_forward_p(const tnn_grid_desc *d, const GridLevels &lv, const GridParams &gp, const float *x, const float4 *order,
                                  const void *table, void *out, int out_dtype, size_t M, hipStream_t s) {
-    if (d->param_dtype == TNN_FP32) return launch_grid_forward_o<D, F, float>(lv, gp, x, table, out, out_dtype, M, s);
-    return launch_grid_forward_o<D, F, fp16_t>(lv, gp, x, table, out, out_dtype, M, s);
+    if (d->param_dtype == TNN_FP32) return launch_grid_forward_o<D, F, float>(lv, gp, x, order, table, out, out_dtype, M, s);
+    return launch_grid_forward_o<D, F, fp16_t>(lv, gp, x, order, table, out, out_dtype, M, s);
 }
 
 template <int D, int F, typename TAB>
@@ -474,7 +501,20 @@ TNN_API int tnn_grid_forward(const tnn_grid_desc *desc, const float *d_x, const 
     int rc = grid_common(desc, padded_width, M, &lv, &gp);
     if (rc) return rc;
     if (!d_x || !d_table || !d_out) return fail(TNN_ERR_INVALID_ARGUMENT, "NULL pointer argument");
-    TNN_DISPATCH_DF(desc, rc = (launch_grid_forward_p<D_, F_>(desc, lv, gp, d_x, d_table, d_out, out_dtype, M, as_stream(stream))));
+    TNN_DISPATCH_DF(desc, rc = (launch_grid_forward_p<D_, F_>(desc, lv, gp, d_x, nullptr, d_table, d_out, out_dtype, M, as_stream(stream))));
+    return rc;
+}
+
+TNN_API int tnn_grid_forward_ordered(const tnn_grid_desc *desc, const void *d_order, const void *d_table, void *d_out, int out_dtype,
+                                     uint32_t padded_width, size_t M, tnn_stream_t stream) {
+    GridLevels lv;
+    GridParams gp;
+    int rc = grid_common(desc, padded_width, M, &lv, &gp);
+    if (rc) return rc;
+    if (!d_order || !d_table || !d_out) return fail(TNN_ERR_INVALID_ARGUMENT, "NULL pointer argument");
+    if (reinterpret_cast<uintptr_t>(d_order) & 15) return fail(TNN_ERR_INVALID_ARGUMENT, "d_order must be 16-byte aligned");
+    TNN_DISPATCH_DF(desc, rc = (launch_grid_forward_p<D_, F_>(desc, lv, gp, nullptr, static_cast<const float4 *>(d_order), d_table, d_out,
+                                                              out_dtype, M, as_stream(stream))));
     return rc;
 }
 

@@ -140,6 +140,21 @@ class Harness:
         _lib.check(self.lib.tnn_grid_forward(ctypes.byref(d), ptr(x_t), ptr(table_t), ptr(out), out_dtype, padded_width, M, self.stream()))
         return out
 
+    def grid_order(self, d, x_t):
+        """Cell order of the points: the buffer tnn_grid_forward_ordered reads (records first, then scratch)."""
+        M = x_t.shape[0]
+        nbytes = self.lib.tnn_grid_order_bytes(ctypes.byref(d), M)
+        buf = torch.empty(nbytes, dtype=torch.uint8, device=self.dev)
+        _lib.check(self.lib.tnn_grid_order_points(ctypes.byref(d), ptr(x_t), M, ptr(buf), nbytes, self.stream()))
+        return buf
+
+    def grid_forward_ordered(self, d, order_t, table_t, padded_width, M, out_dtype=FP32, out=None):
+        if out is None:
+            out = torch.full((M, padded_width), float("nan"), dtype=TORCH_DT[out_dtype], device=self.dev)
+        _lib.check(self.lib.tnn_grid_forward_ordered(ctypes.byref(d), ptr(order_t), ptr(table_t), ptr(out), out_dtype, padded_width, M,
+                                                     self.stream()))
+        return out
+
     def grid_mlp_inference(self, gd, desc, x_t, table_t, prep_fwd):
         M = x_t.shape[0]
         y = torch.full((M, desc.width), float("nan"), dtype=TORCH_DT[desc.dtype], device=self.dev)

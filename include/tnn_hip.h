@@ -324,6 +324,10 @@ int tnn_grid_indices(const tnn_grid_desc *desc, const float *d_x, uint32_t *d_in
  * buffer. d_y: M x width of mlp->dtype. M: positive multiple of 8. */
 int tnn_grid_mlp_inference(const tnn_grid_desc *grid, const tnn_mlp_desc *mlp, const float *d_x, const void *d_table,
                            const void *d_prepared_fwd, void *d_y, size_t M, tnn_stream_t stream);
+/* tnn_grid_mlp_inference over points in cell order (d_order: the records tnn_grid_order_points wrote): the same rows of d_y,
+ * bit for bit. */
+int tnn_grid_mlp_inference_ordered(const tnn_grid_desc *grid, const tnn_mlp_desc *mlp, const void *d_order, const void *d_table,
+                                   const void *d_prepared_fwd, void *d_y, size_t M, tnn_stream_t stream);
 /* TNN_OK when tnn_grid_mlp_inference runs this pair of shapes, otherwise the status (and tnn_last_error the reason) it
  * would return: lets a caller choose between the fused call and the two calls once, when the modules are built. */
 int tnn_grid_mlp_supported(const tnn_grid_desc *grid, const tnn_mlp_desc *mlp);

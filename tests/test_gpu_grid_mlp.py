@@ -41,7 +41,10 @@ def chain_and_fused(tnn, cfg, table_dtype, dtype, W, n_hidden, act, out_act, M, 
     enc = tnn.grid_forward(gd, x, table, W, dtype)
     y_chain = tnn.inference(desc, pf, enc)
     y_fused = tnn.grid_mlp_inference(gd, desc, x, table, pf)
+    # the same kernel over the points in cell order writes the same rows
+    y_ordered = tnn.grid_mlp_inference_ordered(gd, desc, tnn.grid_order(gd, x), table, pf, M)
     tnn.sync()
+    assert same_bits(y_ordered, y_fused), "cell order changed the fused kernel's result"
     return dict(gd=gd, table=table, x=x, w=w, desc=desc, enc=enc, y_chain=y_chain, y_fused=y_fused)
 
 

@@ -4,9 +4,9 @@
 
 namespace tnn {
 int grid_mlp_launch_bf16(const tnn_grid_desc *g, const GridLevels &lv, const GridParams &gp, const tnn_mlp_desc *mlp, const float *x,
-                         const void *table, const void *wprep, void *y, size_t M, hipStream_t s);
+                         const float4 *order, const void *table, const void *wprep, void *y, size_t M, hipStream_t s);
 int grid_mlp_launch_fp16(const tnn_grid_desc *g, const GridLevels &lv, const GridParams &gp, const tnn_mlp_desc *mlp, const float *x,
-                         const void *table, const void *wprep, void *y, size_t M, hipStream_t s);
+                         const float4 *order, const void *table, const void *wprep, void *y, size_t M, hipStream_t s);
 } // namespace tnn
 
 using namespace tnn;
@@ -32,16 +32,30 @@ TNN_API int tnn_grid_mlp_supported(const tnn_grid_desc *grid, const tnn_mlp_desc
     return fused_shape_check(grid, mlp, 8, &lv, &gp);
 }
 
-TNN_API int tnn_grid_mlp_inference(const tnn_grid_desc *grid, const tnn_mlp_desc *mlp, const float *d_x, const void *d_table,
-                                   const void *d_prepared_fwd, void *d_y, size_t M, tnn_stream_t stream) {
+static int grid_mlp_any(const tnn_grid_desc *grid, const tnn_mlp_desc *mlp, const float *d_x, const void *d_order, const void *d_table,
+                        const void *d_prepared_fwd, void *d_y, size_t M, tnn_stream_t stream) {
     GridLevels lv;
     GridParams gp;
     int rc = fused_shape_check(grid, mlp, M ? M : 8, &lv, &gp);
     if (rc) return rc;
     // include/network/SwiftNetMLP.h:293-300: the batch must be a multiple of 8
     if (M == 0 || (M % 8) != 0) return fail(TNN_ERR_INVALID_ARGUMENT, "batch size %zu is not a positive multiple of 8", M);
-    if (!d_x || !d_table || !d_prepared_fwd || !d_y) return fail(TNN_ERR_INVALID_ARGUMENT, "NULL pointer argument");
+    if ((!d_x && !d_order) || !d_table || !d_prepared_fwd || !d_y) return fail(TNN_ERR_INVALID_ARGUMENT, "NULL pointer argument");
+    if (reinterpret_cast<uintptr_t>(d_order) & 15) return fail(TNN_ERR_INVALID_ARGUMENT, "d_order must be 16-byte aligned");
     hipStream_t s = as_stream(stream);
-    if (mlp->dtype == TNN_BF16) return grid_mlp_launch_bf16(grid, lv, gp, mlp, d_x, d_table, d_prepared_fwd, d_y, M, s);
-    return grid_mlp_launch_fp16(grid, lv, gp, mlp, d_x, d_table, d_prepared_fwd, d_y, M, s);
+    const float4 *order = static_cast<const float4 *>(d_order);
+    if (mlp->dtype == TNN_BF16) return grid_mlp_launch_bf16(grid, lv, gp, mlp, d_x, order, d_table, d_prepared_fwd, d_y, M, s);
+    return grid_mlp_launch_fp16(grid, lv, gp, mlp, d_x, order, d_table, d_prepared_fwd, d_y, M, s);
+}
+
+TNN_API int tnn_grid_mlp_inference(const tnn_grid_desc *grid, const tnn_mlp_desc *mlp, const float *d_x, const void *d_table,
+                                   const void *d_prepared_fwd, void *d_y, size_t M, tnn_stream_t stream) {
+    if (!d_x) return fail(TNN_ERR_INVALID_ARGUMENT, "NULL pointer argument");
+    return grid_mlp_any(grid, mlp, d_x, nullptr, d_table, d_prepared_fwd, d_y, M, stream);
+}
+
+TNN_API int tnn_grid_mlp_inference_ordered(const tnn_grid_desc *grid, const tnn_mlp_desc *mlp, const void *d_order, const void *d_table,
+                                           const void *d_prepared_fwd, void *d_y, size_t M, tnn_stream_t stream) {
+    if (!d_order) return fail(TNN_ERR_INVALID_ARGUMENT, "NULL pointer argument");
+    return grid_mlp_any(grid, mlp, nullptr, d_order, d_table, d_prepared_fwd, d_y, M, stream);
 }

@@ -162,6 +162,12 @@ class Harness:
                                                    self.stream()))
         return y
 
+    def grid_mlp_inference_ordered(self, gd, desc, order_t, table_t, prep_fwd, M):
+        y = torch.full((M, desc.width), float("nan"), dtype=TORCH_DT[desc.dtype], device=self.dev)
+        _lib.check(self.lib.tnn_grid_mlp_inference_ordered(ctypes.byref(gd), ctypes.byref(desc), ptr(order_t), ptr(table_t), ptr(prep_fwd), ptr(y),
+                                                           M, self.stream()))
+        return y
+
     def grid_backward(self, d, x_t, dLdy_t, dy_dtype, grad_t=None, overwrite=True):
         M, pw = dLdy_t.shape
         if grad_t is None:

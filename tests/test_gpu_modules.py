@@ -384,6 +384,26 @@ def test_network_with_grid_encoding_fused_inference(tcnn, dtype, n_dims, grid, b
         sh.network.tnn_module.inference_with_encoding(sh.encoding.tnn_module, torch.rand((8, 3), device=DEVICE))
 
 
+def test_large_batches_take_the_cell_order_route(tcnn):
+    """From 2^19 rows on the grid encoding (alone, and fused with the network) orders the batch by cell first. Row for row the
+    result equals what the same rows give in batches below the threshold."""
+    n = (1 << 19) + 40
+    cfg = {"otype": "HashGrid", "n_levels": 16, "n_features_per_level": 2, "log2_hashmap_size": 17, "base_resolution": 16, "per_level_scale": 1.447}
+    torch.manual_seed(5)
+    model = tcnn.NetworkWithInputEncoding(3, 4, net_config(64, 2), cfg, dtype=torch.float16, use_bias=False)
+    with torch.no_grad():
+        model.encoding.params.copy_(torch.rand_like(model.encoding.params) * 2 - 1)
+    model.eval()
+    x = torch.rand((n, 3), device=DEVICE)
+    with torch.no_grad():
+        big = model(x)
+        enc_big = model.encoding(x)
+        for lo in (0, 250000, n - 1000):
+            assert torch.equal(model(x[lo:lo + 1000]).view(torch.int16), big[lo:lo + 1000].view(torch.int16))
+            assert torch.equal(model.encoding(x[lo:lo + 1000]), enc_big[lo:lo + 1000])
+    assert float(big.float().abs().max()) > 1e-3
+
+
 def test_nerf_style_directional_network(tcnn):
     """test/python/test_nerf_settings.py:80-86 of the reference: spherical harmonics of degree 4 feeding a network."""
     model = tcnn.NetworkWithInputEncoding(3, 3, net_config(64, 2), {"otype": "SphericalHarmonics", "degree": 4}, dtype=torch.bfloat16)

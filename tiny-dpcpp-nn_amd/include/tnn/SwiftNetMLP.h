@@ -65,8 +65,19 @@ template <typename T, int WIDTH> class SwiftNetMLP : public Network<T> {
                                                 DeviceMatricesView<T> output) {
         if (Network<T>::get_input_width() != WIDTH) throw std::invalid_argument("The encoding must be padded to the network width.");
         const tnn_mlp_desc d = desc();
-        tnn::abi_check(tnn_grid_mlp_inference(&grid, &d, positions, table, this->prepared_forward(), output.GetMatrixPointer(0), M,
-                                              this->get_queue().abi()));
+        if (M >= (size_t(1) << 19)) {
+            // large batches: points in cell order gather from shared lines of the table (same rows, bit for bit)
+            const size_t bytes = tnn_grid_order_bytes(&grid, M);
+            if (!m_grid_order || m_grid_order->size() * sizeof(float) < bytes)
+                m_grid_order = std::make_unique<DeviceMatrix<float>>((bytes + sizeof(float) - 1) / sizeof(float), 1, this->get_queue());
+            tnn::abi_check(tnn_grid_order_points(&grid, positions, M, m_grid_order->data(), m_grid_order->size() * sizeof(float),
+                                                 this->get_queue().abi()));
+            tnn::abi_check(tnn_grid_mlp_inference_ordered(&grid, &d, m_grid_order->data(), table, this->prepared_forward(),
+                                                          output.GetMatrixPointer(0), M, this->get_queue().abi()));
+        } else {
+            tnn::abi_check(tnn_grid_mlp_inference(&grid, &d, positions, table, this->prepared_forward(), output.GetMatrixPointer(0), M,
+                                                  this->get_queue().abi()));
+        }
         return {tnn::event(this->get_queue().get())};
     }
 
@@ -196,6 +207,7 @@ template <typename T, int WIDTH> class SwiftNetMLP : public Network<T> {
     Activation m_output_activation;
     void *workspace_ = nullptr;
     size_t workspace_bytes_ = 0;
+    std::unique_ptr<DeviceMatrix<float>> m_grid_order; // inference_with_grid: the last large batch in cell order
 };
 
 template <typename T, int WIDTH>

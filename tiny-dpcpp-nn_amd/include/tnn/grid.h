@@ -80,8 +80,21 @@ template <typename T> class GridEncodingTemplated : public GridEncoding<T> {
         if (input.n() != this->get_input_width()) throw std::invalid_argument("Dimension mismatch grid encoding forw_impl input");
         if (input.stride() != input.n() || output->stride() != output->n()) throw std::invalid_argument("Only dense matrices are supported.");
         check_max_level();
+        const size_t batch = input.m();
+        if (batch >= kCellOrderMinBatch) {
+            // large batches: order the points by cell first, so that neighbouring lanes gather from the same lines of the
+            // table (same rows, bit for bit; the buffer only grows)
+            const size_t bytes = tnn_grid_order_bytes(&m_desc, batch);
+            if (!m_order || m_order->size() * sizeof(float) < bytes)
+                m_order = std::make_unique<DeviceMatrix<float>>((bytes + sizeof(float) - 1) / sizeof(float), 1, this->get_queue());
+            tnn::abi_check(tnn_grid_order_points(&m_desc, input.GetPointer(), batch, m_order->data(), m_order->size() * sizeof(float),
+                                                 this->get_queue().abi()));
+            tnn::abi_check(tnn_grid_forward_ordered(&m_desc, m_order->data(), this->get_params()->data(), output->GetPointer(), TNN_FP32,
+                                                    this->get_padded_output_width(), batch, this->get_queue().abi()));
+            return nullptr;
+        }
         tnn::abi_check(tnn_grid_forward(&m_desc, input.GetPointer(), this->get_params()->data(), output->GetPointer(), TNN_FP32,
-                                        this->get_padded_output_width(), input.m(), this->get_queue().abi()));
+                                        this->get_padded_output_width(), batch, this->get_queue().abi()));
         return nullptr; // enqueued on the encoding's in-order stream; the caller waits on the queue when it needs the host to see it
     }
 
@@ -123,7 +136,10 @@ template <typename T> class GridEncodingTemplated : public GridEncoding<T> {
         if (this->m_max_level < (float)m_desc.n_levels) throw std::invalid_argument("GridEncoding: max_level below the level count is not supported.");
     }
 
+    static constexpr size_t kCellOrderMinBatch = size_t(1) << 19; // below this the ordering costs what it saves
+
     tnn_grid_desc m_desc;
+    std::unique_ptr<DeviceMatrix<float>> m_order; // records of the last large batch in cell order
     uint32_t m_n_features;
     uint32_t m_n_features_per_level;
     GridOffsetTable m_offset_table;

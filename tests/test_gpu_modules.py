@@ -384,6 +384,34 @@ def test_network_with_grid_encoding_fused_inference(tcnn, dtype, n_dims, grid, b
         sh.network.tnn_module.inference_with_encoding(sh.encoding.tnn_module, torch.rand((8, 3), device=DEVICE))
 
 
+def test_parameters_are_pushed_when_they_change(tcnn):
+    """forward() refreshes the native module's copy of the parameters when `params` changed since the last push: an
+    optimizer step, copy_() and a replaced Parameter are all seen; a write through `.data` needs an explicit set_params()."""
+    torch.manual_seed(11)
+    net = tcnn.Network(8, 4, net_config(32, 2), dtype=torch.bfloat16)
+    x = torch.rand((64, 8), device=DEVICE)
+    opt = torch.optim.Adam(net.parameters(), lr=1e-2)
+    net.train()
+    y0 = net(x)
+    y0.float().square().sum().backward()
+    opt.step()
+    y1 = net(x)
+    assert not torch.equal(y0, y1), "the optimizer step did not reach the kernels"
+    y1b = net(x)
+    assert torch.equal(y1, y1b)
+    state = net._pushed
+    net(x)
+    assert net._pushed == state, "nothing changed, nothing is pushed again"
+    with torch.no_grad():
+        net.params.copy_(torch.zeros_like(net.params))
+    assert float(net(x).detach().float().abs().max()) == 0.0, "copy_() into params did not reach the kernels"
+    net.params.data.fill_(0.01)  # invisible to the version counter
+    net.set_params()
+    assert float(net(x).detach().float().abs().max()) > 0.0
+    net.params = torch.nn.Parameter(torch.zeros_like(net.params))
+    assert float(net(x).detach().float().abs().max()) == 0.0, "a replaced Parameter did not reach the kernels"
+
+
 def test_large_batches_take_the_cell_order_route(tcnn):
     """From 2^19 rows on the grid encoding (alone, and fused with the network) orders the batch by cell first. Row for row the
     result equals what the same rows give in batches below the threshold."""

@@ -1,327 +1,284 @@
-"""torch.nn.Module front end: Network, Encoding, NetworkWithInputEncoding.
+"""torch.nn.Module front end of the MI355X implementation: Network, Encoding, NetworkWithInputEncoding.
 
-Mirrors dpcpp_bindings/tiny_dpcpp_nn/modules.py of the reference: the autograd function (:65-136), the common
-Module base with `.params`, `set_params`, `get_params`, `forward` (:139-261), Network (:264-307), Encoding
-(:309-354) and NetworkWithInputEncoding (:357-421). Same constructor arguments, attributes, padding rules
-(batch to a multiple of 8, network input to the network width with `use_bias` as the fill value) and loss-scale
-handling. The device is PyTorch-ROCm's "cuda" device where the reference uses "xpu".
+The public surface is the reference's (dpcpp_bindings/tiny_dpcpp_nn/modules.py: autograd function :65-136, Module base
+:139-261, Network :264-307, Encoding :309-354, NetworkWithInputEncoding :357-421): the same class names, constructor
+arguments and attributes (`params`, `tnn_module`, `n_input_dims`, `n_output_dims`, `width`, `n_hidden_layers`,
+`loss_scale`, ...), the same padding rules (batch rows to a multiple of 8; network input columns to the network width,
+filled with ones when `use_bias` and zeros otherwise), the same loss scaling (128 for fp16, 1 for bf16) and the same
+layout conventions (`params` of a network is the packed layout, `set_params(tensor)` takes unpacked matrices). The device
+is PyTorch-ROCm's "cuda" where the reference has "xpu".
 
-All compute goes through the extension module `tiny_dpcpp_nn_pybind_module` (HIP kernels); importing this file
-fails if that module is not built. There is no PyTorch fallback.
+Differences in behaviour, all of them savings: the native module's copy of the parameters is refreshed when `params` has
+changed since it was last pushed (PyTorch's version counter), not on every forward; and in evaluation mode under
+`torch.no_grad()` a grid encoding and its network run as one kernel.
+
+All compute goes through the extension module `tiny_dpcpp_nn_pybind_module` (HIP kernels); importing this file fails if it
+is not built. There is no PyTorch fallback.
 """
 import torch
+import torch.nn.functional as F
 
 from .tiny_dpcpp_nn_pybind_module import Activation, create_encoding, create_network
 
-MIN_BATCH_SIZE = 8  # the kernels need the batch size to be a multiple of 8
-
+MIN_BATCH_SIZE = 8  # the kernels take batches that are multiples of 8 rows
 DEFAULT_DEVICE = "cuda"
+
+_ACTIVATIONS = {"relu": Activation.ReLU, "tanh": Activation.Tanh, "sigmoid": Activation.Sigmoid, "linear": Activation.Linear,
+                "none": Activation.Linear}
+_NETWORK_DTYPES = (torch.float16, torch.bfloat16)
 
 
 def free_temporary_memory():
-    """Kept for interface compatibility; the workspaces are owned by the modules."""
+    """Nothing to free: every workspace belongs to a module and goes with it. Kept because callers of the reference call it."""
+
+
+def get_dpcpp_activation(name):
+    try:
+        return _ACTIVATIONS[name.lower()]
+    except KeyError:
+        raise NotImplementedError(f"Activation: {name} not defined") from None
 
 
 def unpad_tensor_to_input_dim(padded_tensor, output_dim):
-    _, current_width = padded_tensor.shape
-    if output_dim > current_width:
+    if output_dim > padded_tensor.shape[1]:
         raise ValueError("input_dim must be less than or equal to the current width of the tensor")
     return padded_tensor[:, :output_dim]
 
 
-def get_dpcpp_activation(name):
-    key = name.lower()
-    if key == "relu":
-        return Activation.ReLU
-    if key == "tanh":
-        return Activation.Tanh
-    if key == "sigmoid":
-        return Activation.Sigmoid
-    if key in ("linear", "none"):
-        return Activation.Linear
-    raise NotImplementedError(f"Activation: {name} not defined")
-
-
 def to_packed_layout_coord(idx, rows, cols):
-    i, j = divmod(idx, cols)
-    if i % 2 == 0:
-        return i * cols + 2 * j
-    return (i - 1) * cols + 2 * j + 1
+    """Flat index of row-major element `idx` of a rows x cols matrix in the packed parameter layout, where the two rows of
+    a pair are interleaved element by element."""
+    row, col = divmod(idx, cols)
+    return (row & ~1) * cols + 2 * col + (row & 1)
 
 
 def from_packed_layout_coord(idx, rows, cols):
-    i, j = divmod(idx, cols * 2)
-    if j % 2 == 0:
-        return (i * 2) * cols + j // 2
-    return (i * 2 + 1) * cols + (j - 1) // 2
+    """Inverse of to_packed_layout_coord."""
+    pair, within = divmod(idx, 2 * cols)
+    return (2 * pair + (within & 1)) * cols + within // 2
 
 
-class _module_function(torch.autograd.Function):
-    @staticmethod
-    def forward(ctx, native_tnn_module, input, params, info, loss_scale):
-        batch_size = input.shape[0]
-        if info["is_in_eval_mode"]:
-            output = native_tnn_module.inference(input)
-        else:
-            output = native_tnn_module.fwd(input)
-        if batch_size > 0:
-            output = output.reshape(batch_size, -1)
+def _rows_padded(n):
+    return -(-n // MIN_BATCH_SIZE) * MIN_BATCH_SIZE
 
-        ctx.save_for_backward(input, output, params)
-        ctx.info = info
-        ctx.native_tnn_module = native_tnn_module
-        ctx.loss_scale = loss_scale
 
-        if "output_dim" in info:
-            return output[..., : info["output_dim"]]  # the columns beyond output_dim are padding
-        return output  # encodings
+def _pad_rows(x, rows):
+    return x if x.shape[0] == rows else F.pad(x, [0, 0, 0, rows - x.shape[0]])
+
+
+class _NativeCall(torch.autograd.Function):
+    """One call into the native module, with the gradients the reference's autograd function returns: for a network, dL/dx
+    (only if asked for) and the weight gradients in the packed layout; for an encoding, the gradient of its table."""
 
     @staticmethod
-    def backward(ctx, doutput):
-        input, _, params = ctx.saved_tensors
-        loss_scale = ctx.loss_scale
+    def forward(ctx, owner, x, params):
+        native = owner.tnn_module
+        y = native.fwd(x) if owner.training else native.inference(x)
+        if x.shape[0] > 0:
+            y = y.reshape(x.shape[0], -1)
+        ctx.owner = owner
+        ctx.save_for_backward(x, params)
+        visible = owner._visible_output_columns()
+        return y if visible is None else y[..., :visible]  # the rest of a network's output row is padding
 
-        if "width" in ctx.info and doutput.shape[1] < ctx.info["width"]:
-            doutput = torch.nn.functional.pad(doutput, [0, ctx.info["width"] - doutput.shape[1]])  # zeros for the padding columns
-
-        batch_size = input.shape[0]
-        # loss scaling: 1 for bf16, where the two passes over the gradient (here and after the kernels) are skipped
-        doutput = (doutput if loss_scale == 1.0 else doutput * loss_scale).contiguous()
+    @staticmethod
+    def backward(ctx, dy):
+        owner = ctx.owner
+        x, params = ctx.saved_tensors
+        scale = owner.loss_scale
+        full = owner._native_output_columns()
+        if full is not None and dy.shape[1] < full:
+            dy = F.pad(dy, [0, full - dy.shape[1]])  # nothing flows back through the padding columns
+        if scale != 1.0:
+            dy = dy * scale  # fp16: keep the deltas clear of the denormal range inside the kernels
+        dy = dy.contiguous()
+        dx = None
         with torch.no_grad():
-            if "encoding_config" in ctx.info:
-                input_grad = None
-                if batch_size == 0:
-                    grad = torch.zeros_like(params)
-                else:
-                    # parameters of encodings are not packed; no gradient w.r.t. the input
-                    _, grad = ctx.native_tnn_module.bwd_with_encoding_grad(doutput, input, False, False)
+            if x.shape[0] == 0:
+                dparams = torch.zeros_like(params)
+                if owner._is_network:
+                    dx = torch.zeros_like(x)
+            elif owner._is_network:
+                # weight gradients packed into the parameter layout; dL/dx costs a product with the first matrix and a
+                # batch-sized store, so it is asked for only when autograd wants it
+                dx, dparams = owner.tnn_module.bwd_no_encoding_grad(dy, True, bool(ctx.needs_input_grad[1]))
+                if dx is not None:
+                    dx = dx.reshape(x.shape[0], -1)
             else:
-                if batch_size == 0:
-                    input_grad, grad = torch.zeros_like(input), torch.zeros_like(params)
-                else:
-                    # pack the gradient into the parameter layout; dL/dinput only when autograd asks for it (the product
-                    # with the first matrix and a batch-sized store otherwise serve nobody)
-                    input_grad, grad = ctx.native_tnn_module.bwd_no_encoding_grad(doutput, True, bool(ctx.needs_input_grad[1]))
-                    if input_grad is not None:
-                        input_grad = input_grad.reshape(batch_size, -1)
-
-        if grad is not None:
-            grad = (grad if loss_scale == 1.0 else grad / loss_scale).reshape(params.shape).to(params.dtype)
-        if input_grad is not None and loss_scale != 1.0:
-            input_grad = input_grad / loss_scale
-        # one entry per argument of forward
-        return (None, input_grad, grad, None, None)
+                # a table is not packed, and positions get no gradient
+                _, dparams = owner.tnn_module.bwd_with_encoding_grad(dy, x, False, False)
+        if dparams is not None:
+            if scale != 1.0:
+                dparams = dparams / scale
+            dparams = dparams.reshape(params.shape).to(params.dtype)
+        if dx is not None and scale != 1.0:
+            dx = dx / scale
+        return None, dx, dparams
 
 
 class Module(torch.nn.Module):
-    def __init__(
-        self,
-        dtype,  # float for encodings, half precision for networks
-        device=DEFAULT_DEVICE,
-        store_params_as_full_precision=True,
-        use_bias=True,
-        init_module=True,
-    ):
+    """Base of the three front-end classes: owns the native module (`tnn_module`) and the PyTorch-side parameter tensor
+    `params` (fp32 when `store_params_as_full_precision`, else the module's dtype; a network's is in the packed layout)."""
+
+    _is_network = False
+
+    def __init__(self, dtype, device=DEFAULT_DEVICE, store_params_as_full_precision=True, use_bias=True, init_module=True):
         super().__init__()
+        self.dtype = dtype
         self.device = device
         self.use_bias = use_bias
-        self.dtype = dtype
         self.store_params_as_full_precision = store_params_as_full_precision
         self.loss_scale = 128.0 if dtype == torch.float16 else 1.0
-
+        self._pushed = None  # (tensor identity, storage address, version) of `params` when the native module last took it
         if not init_module:
             return
-
         self.tnn_module = self.create_module()
-
-        if self.tnn_module.n_params():
-            initial_params = self.tnn_module.initial_params()
-            params_dtype = torch.float32 if self.store_params_as_full_precision else self.dtype
-            # memory owned by PyTorch, independent of the arrays inside the native module
-            self.params = torch.nn.Parameter(initial_params.clone().detach().to(params_dtype), requires_grad=True)
-        else:
+        if self.tnn_module.n_params() == 0:
             print("No params initialised, as n_params = 0. This is correct for Encodings (apart from grid encodings).")
             self.params = torch.nn.Parameter(torch.zeros(1, device=self.device), requires_grad=False)
+            return
+        held = torch.float32 if store_params_as_full_precision else dtype
+        # PyTorch's own memory, not a view of the native module's arrays
+        self.params = torch.nn.Parameter(self.tnn_module.initial_params().detach().clone().to(held), requires_grad=True)
+
+    # ---- what the autograd function asks of its owner ------------------------------------------------------------
+    def _visible_output_columns(self):
+        return None
+
+    def _native_output_columns(self):
+        return None
+
+    # ---- parameters ----------------------------------------------------------------------------------------------
+    def _params_state(self):
+        p = self.params
+        return (id(p), p.data_ptr(), p._version)
+
+    def _push(self, tensor, packed):
+        t = tensor.detach()
+        # a network on the GPU converts fp32 / fp16 / bf16 to its own type in the kernel that copies; everything else is cast here
+        if not (self._is_network and t.is_cuda and t.dtype in (torch.float32,) + _NETWORK_DTYPES):
+            t = t.to(self.dtype)
+        self.tnn_module.set_params(t.contiguous(), packed)
 
     def set_params(self, params=None):
-        """params given: a flat tensor of unpacked [in][out] matrices (networks) or the table (encodings).
-        params None: push `self.params`, which already is in the native (packed) layout."""
-        if not self.tnn_module.n_params():
+        """`params` given: a flat tensor of unpacked [in][out] matrices (network) or the table (encoding); it is pushed to the
+        native module and `self.params` takes what the module then holds. `None`: push `self.params` as it is (a network's is
+        already packed). Always pushes; `forward` only does so when `params` has changed."""
+        if self.tnn_module.n_params() == 0:
             if params is not None:
                 raise RuntimeError("Network has no parameters. Cannot set params")
             return
+        if params is None:
+            self._push(self.params, packed=self._is_network)
+        else:
+            assert isinstance(params, torch.Tensor), "Params is not a torch.Tensor"
+            self._push(params, packed=False)
+            with torch.no_grad():
+                self.params.copy_(self.get_params().reshape(self.params.shape))
+        self._pushed = self._params_state()
 
-        pushing_own = params is None
-        packed = pushing_own and self.name != "encoding"  # encoding parameters are never packed
-        if pushing_own:
-            params = self.params
-        assert isinstance(params, torch.Tensor), "Params is not a torch.Tensor"
-
-        pushed = params.detach()
-        if not (pushed.is_cuda and pushed.dtype in (torch.float32, torch.float16, torch.bfloat16) and self.name != "encoding"):
-            pushed = pushed.to(self.dtype)  # a network on the GPU converts to its own type itself, in the kernel that copies
-        self.tnn_module.set_params(pushed.contiguous(), packed)
-
-        if not pushing_own:
-            # keep the Python-side copy equal to what the native module holds (networks: the packed layout). When the
-            # module's own `.params` were pushed the two already agree, and the copy back (a whole table for a grid) is skipped.
-            self.params.data.copy_(self.get_params().reshape(self.params.shape))
+    def _push_if_changed(self):
+        """In-place updates (optimizer steps, copy_, load_state_dict) raise the tensor's version; a replaced tensor has another
+        identity or address. Writes through `.data` do neither: call set_params() after those."""
+        if self.tnn_module.n_params() and self._pushed != self._params_state():
+            self.set_params()
 
     def get_params(self):
-        """The parameters as the native module holds them (networks: packed layout)."""
+        """The parameters as the native module holds them (a network's: packed layout)."""
         return self.tnn_module.get_params()
 
+    # ---- evaluation ----------------------------------------------------------------------------------------------
+    def _prepare_input(self, x):
+        return _pad_rows(x, _rows_padded(x.shape[0])).to(dtype=self.dtype)
+
     def forward(self, x):
-        batch_size, input_dim = x.shape
-        padded_batch_size = (batch_size + MIN_BATCH_SIZE - 1) // MIN_BATCH_SIZE * MIN_BATCH_SIZE
-
-        padded_tensor = x if batch_size == padded_batch_size else torch.nn.functional.pad(x, [0, 0, 0, padded_batch_size - batch_size])
-        padded_tensor = padded_tensor.to(dtype=self.dtype)
-
-        if self.name == "network" and input_dim != self.width:
-            # the bias trick: with use_bias the padding columns hold ones (the native module zeroes the weights
-            # of the columns beyond the next multiple of 16), otherwise zeros
-            padded_tensor = torch.nn.functional.pad(padded_tensor, [0, self.width - input_dim, 0, 0], "constant", float(self.use_bias))
-
-        info = {"is_in_eval_mode": not self.training}
-        if hasattr(self, "n_hidden_layers"):
-            info.update(
-                {
-                    "n_hidden_layers": self.n_hidden_layers - 1,
-                    "input_dim": self.n_input_dims,
-                    "output_dim": self.n_output_dims,
-                    "width": self.width,
-                }
-            )
-        if hasattr(self, "encoding_config"):
-            info.update({"encoding_config": self.encoding_config})
-
-        self.set_params()
-        output = _module_function.apply(self.tnn_module, padded_tensor.contiguous(), self.params, info, self.loss_scale)
-        return output[:batch_size, ...]
+        batch = x.shape[0]
+        self._push_if_changed()
+        y = _NativeCall.apply(self, self._prepare_input(x).contiguous(), self.params)
+        return y[:batch]
 
 
 class Network(Module):
-    def __init__(
-        self,
-        n_input_dims,
-        n_output_dims,
-        network_config,
-        store_params_as_full_precision=True,
-        device=DEFAULT_DEVICE,
-        dtype=torch.float16,
-        use_bias=True,
-    ):
-        assert dtype in (torch.float16, torch.bfloat16), f"Only torch.float16 or torch.bfloat16 supported, got: {dtype}"
-        self.network_config = network_config
-        self.width = self.network_config["n_neurons"]
+    _is_network = True
+    name = "network"
+
+    def __init__(self, n_input_dims, n_output_dims, network_config, store_params_as_full_precision=True, device=DEFAULT_DEVICE,
+                 dtype=torch.float16, use_bias=True):
+        assert dtype in _NETWORK_DTYPES, f"Only torch.float16 or torch.bfloat16 supported, got: {dtype}"
         self.n_input_dims = n_input_dims
         self.n_output_dims = n_output_dims
-        self.n_hidden_layers = self.network_config["n_hidden_layers"]
-        self.activation = get_dpcpp_activation(self.network_config["activation"])
-        self.output_activation = get_dpcpp_activation(self.network_config["output_activation"])
-        self.name = "network"
-        super().__init__(
-            device=device,
-            dtype=dtype,
-            store_params_as_full_precision=store_params_as_full_precision,
-            use_bias=use_bias,
-        )
+        self.network_config = network_config
+        self.width = network_config["n_neurons"]
+        self.n_hidden_layers = network_config["n_hidden_layers"]
+        self.activation = get_dpcpp_activation(network_config["activation"])
+        self.output_activation = get_dpcpp_activation(network_config["output_activation"])
+        super().__init__(dtype=dtype, device=device, store_params_as_full_precision=store_params_as_full_precision, use_bias=use_bias)
 
     def create_module(self):
-        return create_network(
-            self.n_input_dims,
-            self.n_output_dims,
-            self.n_hidden_layers,
-            self.activation,
-            self.output_activation,
-            self.width,
-            str(self.dtype),
-            self.use_bias,
-        )
+        return create_network(self.n_input_dims, self.n_output_dims, self.n_hidden_layers, self.activation, self.output_activation,
+                              self.width, str(self.dtype), self.use_bias)
+
+    def _visible_output_columns(self):
+        return self.n_output_dims
+
+    def _native_output_columns(self):
+        return self.width
+
+    def _prepare_input(self, x):
+        x = super()._prepare_input(x)
+        missing = self.width - x.shape[1]
+        if missing:
+            # the bias trick: ones in the padding columns when use_bias (the native module zeroes the weights of the columns
+            # beyond the next multiple of 16), zeros otherwise
+            x = F.pad(x, [0, missing], "constant", float(self.use_bias))
+        return x
 
 
 class Encoding(Module):
-    def __init__(
-        self,
-        n_input_dims,
-        encoding_config,
-        n_output_dims=None,  # None: the encoding's own output width
-        device=DEFAULT_DEVICE,
-        dtype=torch.float,
-        store_params_as_full_precision=True,
-    ):
+    name = "encoding"
+
+    def __init__(self, n_input_dims, encoding_config, n_output_dims=None, device=DEFAULT_DEVICE, dtype=torch.float,
+                 store_params_as_full_precision=True):
         assert dtype == torch.float, "Only torch.float is currently supported for encoding (the grid gradients are float atomics)"
         self.n_input_dims = n_input_dims
         self.encoding_config = encoding_config
-        self.padded_output_dims = n_output_dims
-        self.encoding_name = self.encoding_config["otype"]
-        self.name = "encoding"
-
-        if "n_dims_to_encode" not in self.encoding_config:
-            self.encoding_config["n_dims_to_encode"] = self.n_input_dims
-
-        super().__init__(device=device, dtype=dtype, store_params_as_full_precision=store_params_as_full_precision)
-
-        # only known once the native module exists
-        self.n_output_dims = self.tnn_module.n_output_dims()
+        self.encoding_config.setdefault("n_dims_to_encode", n_input_dims)
+        self.encoding_name = encoding_config["otype"]
+        self.padded_output_dims = n_output_dims  # None: the encoding's own width
+        super().__init__(dtype=dtype, device=device, store_params_as_full_precision=store_params_as_full_precision)
+        self.n_output_dims = self.tnn_module.n_output_dims()  # known once the native module exists
 
     def create_module(self):
         return create_encoding(self.encoding_name, self.encoding_config, self.padded_output_dims)
 
 
 class NetworkWithInputEncoding(Module):
-    def __init__(
-        self,
-        n_input_dims,
-        n_output_dims,
-        network_config,
-        encoding_config,
-        device=DEFAULT_DEVICE,
-        store_params_as_full_precision=True,
-        dtype=torch.float16,
-        use_bias=True,
-    ):
-        assert dtype in (torch.float16, torch.bfloat16), (
-            f"Only torch.float16 or torch.bfloat16 supported, got: {dtype}."
-            " Note, that dtype here only refers to dtype of Network, the Encoding is always float."
-        )
-        super().__init__(dtype=dtype, init_module=False)
+    name = "network_with_encoding"
 
-        self.encoding_config = encoding_config
-        self.network_config = network_config
-        self.width = self.network_config["n_neurons"]
+    def __init__(self, n_input_dims, n_output_dims, network_config, encoding_config, device=DEFAULT_DEVICE,
+                 store_params_as_full_precision=True, dtype=torch.float16, use_bias=True):
+        assert dtype in _NETWORK_DTYPES, (f"Only torch.float16 or torch.bfloat16 supported, got: {dtype}."
+                                          " Note, that dtype here only refers to dtype of Network, the Encoding is always float.")
+        super().__init__(dtype=dtype, init_module=False)
         self.n_input_dims = n_input_dims
         self.n_output_dims = n_output_dims
-        self.n_hidden_layers = self.network_config["n_hidden_layers"]
-        self.activation = get_dpcpp_activation(self.network_config["activation"])
-        self.output_activation = get_dpcpp_activation(self.network_config["output_activation"])
-        self.name = "network_with_encoding"
-
-        self.encoding = Encoding(
-            n_input_dims,
-            encoding_config,
-            device=device,
-            dtype=torch.float,
-            store_params_as_full_precision=store_params_as_full_precision,
-            n_output_dims=network_config["n_neurons"],
-        )
-        assert self.encoding.n_output_dims == network_config["n_neurons"]
-        self.network = Network(
-            self.encoding.n_output_dims,
-            n_output_dims,
-            network_config,
-            device=device,
-            dtype=dtype,
-            store_params_as_full_precision=store_params_as_full_precision,
-            use_bias=use_bias,
-        )
+        self.network_config = network_config
+        self.encoding_config = encoding_config
+        self.width = network_config["n_neurons"]
+        self.n_hidden_layers = network_config["n_hidden_layers"]
+        self.activation = get_dpcpp_activation(network_config["activation"])
+        self.output_activation = get_dpcpp_activation(network_config["output_activation"])
+        # the encoding pads its rows to the network width itself, so the network never pads its input
+        self.encoding = Encoding(n_input_dims, encoding_config, n_output_dims=self.width, device=device, dtype=torch.float,
+                                 store_params_as_full_precision=store_params_as_full_precision)
+        assert self.encoding.n_output_dims == self.width
+        self.network = Network(self.width, n_output_dims, network_config, store_params_as_full_precision=store_params_as_full_precision,
+                               device=device, dtype=dtype, use_bias=use_bias)
         self.network_with_encoding = torch.nn.Sequential(self.encoding, self.network)
 
     @property
     def params(self):
-        # the network's parameters; the encoding's are reached through `.encoding.params`
-        return self.network.params
+        return self.network.params  # the table is `self.encoding.params`
 
     def get_params(self):
         raise RuntimeError("Not implemented.")
@@ -330,18 +287,17 @@ class NetworkWithInputEncoding(Module):
         self.network.set_params(params)
 
     def forward(self, x):
-        if (not self.training and not torch.is_grad_enabled() and x.shape[0] > 0
-                and self.network.tnn_module.can_fuse_encoding(self.encoding.tnn_module)):
-            return self._fused_inference(x)
-        return self.network_with_encoding(x)
+        one_kernel = (not self.training and not torch.is_grad_enabled() and x.shape[0] > 0
+                      and self.network.tnn_module.can_fuse_encoding(self.encoding.tnn_module))
+        return self._fused_inference(x) if one_kernel else self.network_with_encoding(x)
 
     def _fused_inference(self, x):
-        """Evaluation without autograd on a grid encoding: encoding and network run as one kernel, the encoded matrix is
-        never stored. Same values as the two modules in turn (the reference's only route, modules.py:357-421)."""
-        batch_size = x.shape[0]
-        padded_batch_size = (batch_size + MIN_BATCH_SIZE - 1) // MIN_BATCH_SIZE * MIN_BATCH_SIZE
-        padded = x if batch_size == padded_batch_size else torch.nn.functional.pad(x, [0, 0, 0, padded_batch_size - batch_size])
-        self.encoding.set_params()
-        self.network.set_params()
-        output = self.network.tnn_module.inference_with_encoding(self.encoding.tnn_module, padded.to(torch.float32).contiguous())
-        return output.reshape(padded_batch_size, -1)[:batch_size, : self.n_output_dims]
+        """Evaluation without autograd on a grid encoding: one kernel, the encoded matrix is never stored; the values are those
+        of the two modules in turn (the reference's only route)."""
+        batch = x.shape[0]
+        rows = _rows_padded(batch)
+        self.encoding._push_if_changed()
+        self.network._push_if_changed()
+        positions = _pad_rows(x, rows).to(torch.float32).contiguous()
+        y = self.network.tnn_module.inference_with_encoding(self.encoding.tnn_module, positions)
+        return y.reshape(rows, -1)[:batch, : self.n_output_dims]

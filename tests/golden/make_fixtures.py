@@ -78,6 +78,34 @@ def main():
         open(os.path.join(HERE, "spherical_harmonics_degree4.json"), "w"),
     )
 
+    # include/common/common_device.h:33-206 : the 64 polynomials of sh_enc (bands 0-7), evaluated from the reference's own
+    # text at seeded points. The fixture holds encoding inputs in [0, 1]^3 (the encoding maps them to 2x - 1,
+    # include/encodings/spherical_harmonics.h:38-72) and the 64 values per point.
+    import random
+    import re
+    src = open(os.path.join(REF, "include/common/common_device.h")).read()
+    body = src[src.index("void sh_enc("):src.index("} // namespace kernels") if "} // namespace kernels" in src else len(src)]
+    body = re.sub(r"//[^\n]*", "", body)  # the comments repeat the formulas in another notation
+    stmts = re.findall(r"data_out\[(\d+) \+ offset\]\s*=\s*\(T\)\((.*?)\);", body, flags=re.S)
+    assert [int(i) for i, _ in stmts] == list(range(64)), "expected the 64 assignments of sh_enc in order"
+    exprs = [re.sub(r"(?<=[0-9.])f\b", "", " ".join(e.split())) for _, e in stmts]
+    rnd = random.Random(2024)
+    inputs = [[rnd.random(), rnd.random(), rnd.random()] for _ in range(24)] + [[1.0, 1.0, 1.0], [0.0, 0.5, 1.0], [0.5, 0.5, 0.5]]
+    expected = []
+    for p in inputs:
+        x, y, z = (2.0 * c - 1.0 for c in p)
+        env = dict(x=x, y=y, z=z, xy=x * y, xz=x * z, yz=y * z, x2=x * x, y2=y * y, z2=z * z)
+        env.update(x4=env["x2"] ** 2, y4=env["y2"] ** 2, z4=env["z2"] ** 2)
+        env.update(x6=env["x4"] * env["x2"], y6=env["y4"] * env["y2"], z6=env["z4"] * env["z2"])
+        expected.append([eval(e, {"__builtins__": {}}, env) for e in exprs])
+    json.dump(
+        {
+            "source": "include/common/common_device.h:33-206 (the polynomials of sh_enc, evaluated in double precision)",
+            "degree": 8, "atol": 2.0e-5, "inputs": inputs, "expected": expected,
+        },
+        open(os.path.join(HERE, "spherical_harmonics_degree8.json"), "w"),
+    )
+
 
 if __name__ == "__main__":
     main()

@@ -79,6 +79,14 @@ def test_spherical_harmonics_golden(tnn):
     assert np.allclose(out, [[0.2821, 1.0, 1.0]] * 2, atol=1e-3)
 
 
+def test_spherical_harmonics_all_64_polynomials(tnn):
+    """The GPU kernel, bands 0-7, against the values of the reference's 64 polynomials (include/common/common_device.h:33-206)."""
+    fx = json.load(open(os.path.join(G, "spherical_harmonics_degree8.json")))
+    x = torch.tensor(fx["inputs"], dtype=torch.float32, device=tnn.dev)
+    out = tnn.sh_forward(x, fx["degree"], 64).cpu().numpy()
+    assert np.allclose(out, np.float64(fx["expected"]), atol=fx["atol"], rtol=1e-5)
+
+
 def test_argument_checks(tnn):
     x = torch.zeros((8, 3), device=tnn.dev)
     o = torch.zeros((8, 64), device=tnn.dev)

@@ -412,6 +412,38 @@ def test_parameters_are_pushed_when_they_change(tcnn):
     assert float(net(x).detach().float().abs().max()) == 0.0, "a replaced Parameter did not reach the kernels"
 
 
+def test_modules_follow_the_callers_stream(tcnn):
+    """A module's kernels go to torch's current stream at the time of the call: an input that is still being produced on a
+    side stream is complete when they read it, without any host wait, and a module can move between streams."""
+    torch.manual_seed(2)
+    net = tcnn.Network(64, 64, net_config(64, 2), dtype=torch.bfloat16, use_bias=False)
+    enc = tcnn.Encoding(2, dict(GRID_2D))
+    net.eval()
+    enc.eval()
+    n = 1 << 16
+    base = torch.rand((n, 64), device=DEVICE)
+    pos = torch.rand((n, 2), device=DEVICE)
+    big = torch.rand((4096, 4096), device=DEVICE)
+    with torch.no_grad():
+        want = net((base * 2 - 1)), enc(pos * 0.5)
+        torch.cuda.synchronize()
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(10):
+                busy = big @ big  # keeps the side stream busy while the host runs ahead
+            x = base * 2 - 1 + busy[0, 0] * 0  # produced behind that work, on the side stream
+            p = pos * 0.5 + busy[0, 0] * 0
+            got = net(x), enc(p)
+        side.synchronize()
+        for g, w in zip(got, want):
+            assert torch.equal(g, w)
+        # back on the default stream the module waits for what it left on the side stream by itself
+        again = net(base * 2 - 1)
+        torch.cuda.synchronize()
+        assert torch.equal(again, want[0])
+
+
 def test_large_batches_take_the_cell_order_route(tcnn):
     """From 2^19 rows on the grid encoding (alone, and fused with the network) orders the batch by cell first. Row for row the
     result equals what the same rows give in batches below the threshold."""

@@ -90,6 +90,19 @@ def test_sh_recurrence_equals_the_references_expressions(oracle):
             assert abs(out[i, idx] - val) <= 2e-6 * max(1.0, abs(val)), (idx, out[i, idx], val)
 
 
+def test_sh_all_64_polynomials_of_the_reference(oracle):
+    """Bands 0-7 against the values of the reference's 64 spelled-out polynomials (include/common/common_device.h:33-206) at
+    seeded points, so that a slipped sign or normalisation in the higher bands fails here and not only at the user."""
+    fx = json.load(open(os.path.join(G, "spherical_harmonics_degree8.json")))
+    x = np.float32(fx["inputs"])
+    out = oracle.sh_forward(fx["degree"], x, 64)
+    ref = np.float64(fx["expected"])
+    assert out.shape == ref.shape == (len(x), 64)
+    assert np.allclose(out, ref, atol=fx["atol"], rtol=1e-5)
+    # every band is present in the check: no column of the expected values is (near) constant zero
+    assert (np.abs(ref).max(axis=0) > 1e-3).all()
+
+
 def test_sh_orthonormal_on_the_sphere(oracle):
     """All 64 functions are orthonormal under the surface integral (Gauss-Legendre in cos(theta) x uniform in phi)."""
     n_t, n_p = 24, 48

@@ -120,6 +120,7 @@ class queue {
     queue() = default;
     explicit queue(hipStream_t s) : stream_(s) {}
     hipStream_t get() const { return stream_; }
+    void rebind(hipStream_t s) { stream_ = s; } // every holder of a reference to this queue follows
     tnn_stream_t abi() const { return reinterpret_cast<tnn_stream_t>(stream_); }
     void wait() const {
         if (hipStreamSynchronize(stream_) != hipSuccess) throw std::runtime_error("hipStreamSynchronize failed");

@@ -1,8 +1,8 @@
 // The tensor-level module interface that the Python bindings wrap. Mirrors include/tnn_api.h of the reference:
 // tnn::Module (:62-303), EncodingModule<T> (:306-474), NetworkModule<T, WIDTH> (:477-697). Tensors are
-// PyTorch-ROCm tensors on the GPU; the stream is torch's current HIP stream at construction (the reference takes
-// the current XPU stream's queue, :295-302). Results are handed back as fresh torch allocations (clones of the
-// module's grow-only workspaces), and every method blocks until its work is done, as in the reference.
+// PyTorch-ROCm tensors on the GPU; every method runs on torch's current HIP stream at the time of the call (the
+// reference takes the current XPU stream's queue, :295-302). Results are handed back as fresh torch allocations; the
+// work is ordered with the caller's tensor operations by the stream, so no method makes the host wait.
 #pragma once
 
 #include <c10/hip/HIPStream.h>
@@ -62,12 +62,28 @@ class Module {
 
     tnn::queue &get_queue() { return queue_; }
 
-    /// The reference blocks at the end of every method. Here the module's work and the tensor operations of the caller
-    /// share one in-order stream (torch's current stream, taken at construction), so the results are ordered without a
-    /// host wait; only when the caller has moved to another stream since does the method wait for the module's own.
-    void finish() {
-        if (c10::hip::getCurrentHIPStream().stream() != queue_.get()) queue_.wait();
+    /// First thing in every method: the module's kernels go to the stream the caller's tensor operations are on, so inputs
+    /// produced there are complete when the kernels read them and the tensors handed back (allocated from that stream's
+    /// pool) are written on it. When the caller has changed streams since the last call, the new stream first waits for
+    /// what the module still has in flight on the old one (its workspaces and parameter copies are shared between calls).
+    void enter() {
+        const hipStream_t now = c10::hip::getCurrentHIPStream(device_index_).stream();
+        const hipStream_t before = queue_.get();
+        if (now == before) return;
+        hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+        (void)hipStreamIsCapturing(now, &capturing);
+        if (capturing == hipStreamCaptureStatusNone) {
+            hipEvent_t done = nullptr;
+            tnn::hip_check(hipEventCreateWithFlags(&done, hipEventDisableTiming), "hipEventCreateWithFlags");
+            tnn::hip_check(hipEventRecord(done, before), "hipEventRecord");
+            tnn::hip_check(hipStreamWaitEvent(now, done, 0), "hipStreamWaitEvent");
+            tnn::hip_check(hipEventDestroy(done), "hipEventDestroy"); // released once it has completed
+        }
+        queue_.rebind(now);
     }
+
+    /// Nothing to wait for: the call's work is on the caller's stream (the reference blocks here).
+    void finish() {}
 
     template <typename T> static std::vector<T> convertTensorToVector(const torch::Tensor &tensor) {
         const auto cpu = tensor.to(torch::kCPU).to(torch::kFloat32).contiguous();
@@ -125,6 +141,7 @@ template <typename T> class EncodingModule : public Module {
     ~EncodingModule() { this->FreeWorkspace(); }
 
     torch::Tensor forward_pass(const torch::Tensor &input_tensor) override {
+        this->enter();
         CHECK_INPUT(input_tensor);
         TORCH_CHECK(input_tensor.scalar_type() == torch::kFloat32, "input_tensor must be float32");
         const size_t batch_size = input_tensor.sizes()[0];
@@ -150,6 +167,7 @@ template <typename T> class EncodingModule : public Module {
 
     std::tuple<torch::Tensor, torch::Tensor> backward_pass(const torch::Tensor &grad_output, const torch::Tensor &input_from_fwd,
                                                            bool pack_transpose_gradient = false, bool get_dl_dinput = false) override {
+        this->enter();
         if (encoding_->get_n_params() == 0) return {torch::Tensor(), torch::Tensor()};
         CHECK_INPUT(grad_output);
         CHECK_INPUT(input_from_fwd);
@@ -183,11 +201,13 @@ template <typename T> class EncodingModule : public Module {
 
     torch::Tensor initialize_params() override { return get_params(); }
     torch::Tensor initialize_params(const torch::Tensor &tensor) override {
+        this->enter();
         set_params(tensor, false);
         return get_params();
     }
 
     void set_params(const torch::Tensor &params, bool weights_are_packed) override {
+        this->enter();
         if (encoding_->get_params() == nullptr) throw std::runtime_error("no encoding params to set");
         if (weights_are_packed) throw std::runtime_error("Packed weights are not supported in api set params");
         CHECK_INPUT(params);
@@ -198,6 +218,7 @@ template <typename T> class EncodingModule : public Module {
     }
 
     torch::Tensor get_params() override {
+        this->enter();
         if (encoding_->get_params()) return convertDeviceMatrixToTorchTensor<T>(*encoding_->get_params());
         return torch::empty({0});
     }
@@ -259,6 +280,7 @@ template <typename T, int WIDTH> class NetworkModule : public Module {
     ~NetworkModule() { this->FreeWorkspace(); }
 
     torch::Tensor inference(const torch::Tensor &input_tensor) override {
+        this->enter();
         const size_t batch_size = CheckedBatch(input_tensor, network_.get_input_width());
         const int64_t out_w = network_.get_output_width();
         if (batch_size == 0) return torch::empty({0, out_w}, torch::TensorOptions().dtype(torch_type<T>::dtype).device(device()));
@@ -278,6 +300,7 @@ template <typename T, int WIDTH> class NetworkModule : public Module {
     }
 
     torch::Tensor inference_with_encoding(const Module &encoding, const torch::Tensor &positions) override {
+        this->enter();
         const tnn_grid_desc *grid = encoding.grid_descriptor();
         if (!grid || !network_.supports_grid_input(*grid))
             throw std::invalid_argument("inference_with_encoding: this encoding / network pair runs as two calls (" +
@@ -297,6 +320,7 @@ template <typename T, int WIDTH> class NetworkModule : public Module {
     }
 
     torch::Tensor forward_pass(const torch::Tensor &input_tensor) override {
+        this->enter();
         const size_t batch_size = CheckedBatch(input_tensor, network_.get_input_width());
         const int64_t out_w = network_.get_output_width();
         if (batch_size == 0) return torch::empty({0, out_w}, torch::TensorOptions().dtype(torch_type<T>::dtype).device(device()));
@@ -316,6 +340,7 @@ template <typename T, int WIDTH> class NetworkModule : public Module {
 
     std::tuple<torch::Tensor, torch::Tensor> backward_pass(const torch::Tensor &grad_output, bool pack_transpose_gradient,
                                                            bool get_dl_dinput) override {
+        this->enter();
         CHECK_INPUT(grad_output);
         TORCH_CHECK(grad_output.dim() == 2, "grad_output must have two dimensions");
         TORCH_CHECK(grad_output.scalar_type() == torch_type<T>::dtype, "grad_output has the wrong dtype");
@@ -358,8 +383,12 @@ template <typename T, int WIDTH> class NetworkModule : public Module {
     }
 
     torch::Tensor initialize_params() override { return get_params(); }
-    torch::Tensor get_params() override { return convertDeviceMatricesToTorchTensor(network_.get_weights_matrices()); }
+    torch::Tensor get_params() override {
+        this->enter();
+        return convertDeviceMatricesToTorchTensor(network_.get_weights_matrices());
+    }
     torch::Tensor initialize_params(const torch::Tensor &tensor) override {
+        this->enter();
         set_params(tensor, false);
         return initialize_params();
     }
@@ -370,6 +399,7 @@ template <typename T, int WIDTH> class NetworkModule : public Module {
     /// The parameters stay on the device: a GPU tensor of any floating dtype is converted and (if unpacked)
     /// packed there. A CPU tensor takes the reference's route through a host vector.
     void set_params(const torch::Tensor &params, bool weights_are_packed) override {
+        this->enter();
         if ((size_t)params.numel() != n_params())
             throw std::runtime_error("m_weights_matrices nelements: " + std::to_string(n_params()) +
                                      " does not match unpacked_weights size: " + std::to_string(params.numel()) +

@@ -612,14 +612,26 @@ class Bench:
         hyper = (1e-3, 0.9, 0.99, 1e-15)
         k0, k1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
 
+        # points in cell order (ordered inside the step: a trainer draws new points every step) unless --no-cell-order; the
+        # packed scatter has no such route
+        ordered = not args.no_cell_order and not args.packed_scatter
+        order_bytes = lib.tnn_grid_order_bytes(g, M)
+        order = torch.empty(max(order_bytes, 16), dtype=torch.uint8, device=t.dev)
+
         def step(i, time_scatter=False):
-            _lib.check(lib.tnn_grid_forward(g, ptr(x), ptr(table), ptr(enc), FP16, W, M, s))
+            if ordered:
+                _lib.check(lib.tnn_grid_order_points(g, ptr(x), M, ptr(order), order_bytes, s))
+                _lib.check(lib.tnn_grid_forward_ordered(g, ptr(order), ptr(table), ptr(enc), FP16, W, M, s))
+            else:
+                _lib.check(lib.tnn_grid_forward(g, ptr(x), ptr(table), ptr(enc), FP16, W, M, s))
             _lib.check(lib.tnn_mlp_train_step_l2_adam(md, ptr(pf), ptr(pb), ptr(enc), ptr(targets), loss_scale, None, ptr(loss), ptr(master),
                                                       ptr(mw), ptr(vw), i + 1, *hyper, None, ptr(d_enc), M, ptr(ws), ws_bytes, None, s))
             if time_scatter:
                 k0.record()
             if args.packed_scatter:
                 _lib.check(lib.tnn_grid_backward_packed(g, ptr(x), ptr(d_enc), FP16, W, ptr(grad_table), 1, M, s))
+            elif ordered:
+                _lib.check(lib.tnn_grid_backward_ordered(g, ptr(order), ptr(d_enc), FP16, W, ptr(grad_table), 1, M, s))
             else:
                 _lib.check(lib.tnn_grid_backward(g, ptr(x), ptr(d_enc), FP16, W, ptr(grad_table), 1, M, s))
             if time_scatter:
@@ -648,7 +660,8 @@ class Bench:
         ach = bpp * M / (scatter_ms * 1e-3) / 1e9
         roof = {"bound": "hbm", "achieved": ach, "peak": PEAK_HBM, "unit": "GB/s", "frac": ach / PEAK_HBM,
                 "traffic": MEASURED_TRAFFIC_BYTES.get(("grid_train_packed" if args.packed_scatter else "grid_train", lg)),
-                "kernel": "grid_backward_kernel (with the fill of the gradient table in front of it)", "kernel_ms": scatter_ms,
+                "kernel": "grid_backward_kernel (with the fill of the gradient table in front of it)" + (" over points in cell order" if ordered else ""),
+                "kernel_ms": scatter_ms,
                 "algorithmic_bytes_per_launch": bpp * M}
         out = line("hash-grid + fused-MLP training samples/s (2-D, 16x2, log2 19; w64, 2 hidden layers; batch 2^18; whole step with both Adam updates)",
                    "samples/s", "f16",

@@ -297,6 +297,14 @@ int tnn_grid_forward_ordered(const tnn_grid_desc *desc, const void *d_order, con
 int tnn_grid_backward(const tnn_grid_desc *desc, const float *d_x, const void *d_dLdy, int dy_dtype,
                       uint32_t padded_width, float *d_grad_table, int overwrite, size_t M, tnn_stream_t stream);
 
+/* tnn_grid_backward over the records of tnn_grid_order_points instead of d_x (no counterpart in the reference). Thread
+ * groups take the points in cell order and read row `row number` of d_dLdy; neighbouring groups then often add to the same
+ * entry, so runs of equal entries inside a wave are summed in registers and added with one atomic per run. The table
+ * receives the same contributions as from tnn_grid_backward in another order of addition (the reference defines none,
+ * grid.h:215-243). */
+int tnn_grid_backward_ordered(const tnn_grid_desc *desc, const void *d_order, const void *d_dLdy, int dy_dtype,
+                              uint32_t padded_width, float *d_grad_table, int overwrite, size_t M, tnn_stream_t stream);
+
 /* The same scatter into an fp16 gradient table, two features of an entry per packed atomic (global_atomic_pk_add_f16): half
  * as many atomic operations as the fp32 route and half the gradient table; the same number of 32-byte requests at the memory
  * side, which is what bounds the pass, so about the same time. No counterpart in the reference, whose

@@ -115,3 +115,45 @@ def test_config_5_full_size_ordered(tnn, oracle):
     rows = torch.randint(0, M, (4096,), device=tnn.dev, generator=gen)
     ref = oracle.grid_forward(CFG5, table.float().cpu().numpy(), x[rows].cpu().numpy(), 32)
     assert_close(ordered[rows].float().cpu().numpy(), ref, FP16, "config 5 ordered", scale=1e-4)
+
+
+@pytest.mark.parametrize("cfg,pd", [(CFG4, FP16), (CFG5, FP16), (dict(CFG5, n_features_per_level=4, n_levels=8, interpolation="Smoothstep"), FP32),
+                                    (dict(CFG4, grid_type="Dense", n_levels=6, n_features_per_level=1), FP16),
+                                    (dict(CFG5, hash="Prime", n_features_per_level=8, n_levels=4, interpolation="Nearest"), FP16)])
+@pytest.mark.parametrize("kind,M", [("uniform", 2011), ("uniform", 70000), ("clustered", 30001), ("identical", 777), ("uniform", 1)])
+def test_ordered_backward_matches_the_oracle(tnn, oracle, cfg, pd, kind, M):
+    """tnn_grid_backward_ordered: the same contributions as tnn_grid_backward, summed per run of equal entries inside a wave
+    first. fp32 sums in another order against the oracle's double sum: |err| <= 1e-5 x the largest entry (the bar of the
+    plain call); identical points make runs of 16 in every wave and clustered ones runs of every length."""
+    D, F, L = cfg["n_dims"], cfg["n_features_per_level"], cfg["n_levels"]
+    rng = np.random.default_rng(M + 31 * D + F)
+    x = points(kind, M, D, rng)
+    pw = L * F + 8
+    d = tnn.grid_desc(cfg, pd)
+    n = tnn.grid_n_params(d)
+    xt = torch.from_numpy(x).to(tnn.dev)
+    g = rng.standard_normal((M, pw)).astype(np.float32)
+    gt = torch.from_numpy(g).to(tnn.dev)
+    buf = tnn.grid_order(d, xt)
+    grad = tnn.grid_backward_ordered(d, buf, gt, FP32).cpu().numpy()
+    ref = oracle.grid_backward(cfg, x, g, n)
+    bar = 1e-5 * max(1.0, np.abs(ref).max())
+    assert np.abs(grad - ref).max() <= bar
+    plain = tnn.grid_backward(d, xt, gt, FP32).cpu().numpy()
+    assert np.abs(grad - plain).max() <= 2 * bar
+    # accumulate mode adds on top of what the table holds
+    twice = tnn.grid_backward_ordered(d, buf, gt, FP32, grad_t=torch.from_numpy(grad).to(tnn.dev), overwrite=False).cpu().numpy()
+    assert np.abs(twice - 2 * ref).max() <= 2 * bar
+
+
+def test_ordered_backward_config_4_full_size(tnn, oracle):
+    cfg, M = CFG4, 1 << 18
+    d = tnn.grid_desc(cfg, FP16)
+    n = tnn.grid_n_params(d)
+    gen = torch.Generator(device=tnn.dev).manual_seed(6)
+    x = torch.rand((M, 2), device=tnn.dev, generator=gen)
+    g = (torch.rand((M, 32), device=tnn.dev, generator=gen) - 0.5).to(torch.float16)
+    grad = tnn.grid_backward_ordered(d, tnn.grid_order(d, x), g, FP16).cpu().numpy()
+    ref = oracle.grid_backward(cfg, x.cpu().numpy(), g.to(torch.float32).cpu().numpy(), n)
+    assert np.abs(grad - ref).max() <= 1e-5 * np.abs(ref).max() + 1e-4
+    assert_close(grad, ref, FP32, "gradient table", scale=1e2, frac_ok=1e-4)

@@ -153,8 +153,24 @@ struct BackwardPlan {
     uint8_t big_level[TNN_GRID_MAX_LEVELS];
 };
 
+constexpr int kGridWave = 64;                    // lanes of a wave
 constexpr uint32_t kPrivateLdsBytes = 64 * 1024; // per workgroup; two such workgroups fit a CU
 constexpr uint32_t kPrivateChunk = 4096;         // points per workgroup on the LDS route
+
+// Coordinates and row number of the i-th point: row i of x, or the i-th record of the cell order (grid_order.hip).
+template <int D>
+__device__ __forceinline__ long long load_point(const float *__restrict__ xin, const float4 *__restrict__ order, long long i, float (&x)[D]) {
+    if (order) {
+        const float4 r = order[i];
+        x[0] = r.x;
+        x[1] = r.y;
+        if (D > 2) x[D - 1] = r.z;
+        return (long long)__float_as_uint(r.w);
+    }
+#pragma unroll
+    for (int d = 0; d < D; ++d) x[d] = xin[i * D + d];
+    return i;
+}
 
 // Gradient contributions of one point to one level: visits (entry index, weight) of every corner.
 template <int D, typename Fn>
@@ -216,7 +232,7 @@ template <int F> struct BackwardLanes<F, fp16_t> { static constexpr int FL = F /
 template <int D, int F, typename G, typename GT>
 __global__ void __launch_bounds__(kGridThreads)
     grid_backward_kernel(const GridLevels lv, const GridParams gp, const BackwardPlan bp, const float *__restrict__ xin,
-                         const G *__restrict__ dLdy, GT *__restrict__ grad, long long M) {
+                         const float4 *__restrict__ order, const G *__restrict__ dLdy, GT *__restrict__ grad, long long M) {
     extern __shared__ float priv[];
     const uint32_t n_small_blocks = bp.n_small * bp.small_blocks;
     if (blockIdx.x < n_small_blocks) {
@@ -230,11 +246,10 @@ __global__ void __launch_bounds__(kGridThreads)
         const long long last = first + bp.chunk < M ? first + bp.chunk : M;
         for (long long i = first + threadIdx.x; i < last; i += kGridThreads) {
             float x[D];
-#pragma unroll
-            for (int d = 0; d < D; ++d) x[d] = xin[i * D + d];
+            const long long row = load_point<D>(xin, order, i, x);
             float gy[F];
 #pragma unroll
-            for (int f = 0; f < F; ++f) gy[f] = (float)dLdy[i * gp.padded_width + l * F + f];
+            for (int f = 0; f < F; ++f) gy[f] = (float)dLdy[row * gp.padded_width + l * F + f];
             for_each_corner<D>(x, scale, size, res, flags, gp.hash_type, gp.interpolation, [&](uint32_t idx, float w) {
 #pragma unroll
                 for (int f = 0; f < F; ++f) atomicAdd(&priv[idx * F + f], w * gy[f]);
@@ -262,23 +277,24 @@ __global__ void __launch_bounds__(kGridThreads)
     constexpr int FL = BackwardLanes<F, GT>::FL, LPI = 2 * FL;
     const uint32_t b = blockIdx.x - n_small_blocks;
     const uint32_t l = bp.big_level[b / bp.big_blocks];
-    const long long i = (long long)(b % bp.big_blocks) * (kGridThreads / LPI) + threadIdx.x / LPI;
-    if (i >= M) return;
+    const long long i_raw = (long long)(b % bp.big_blocks) * (kGridThreads / LPI) + threadIdx.x / LPI;
+    const bool live = i_raw < M;
+    if (!live && !order) return;
+    const long long i = live ? i_raw : M - 1; // in cell order every lane stays for the exchange between lanes below
     const int dx = (threadIdx.x % LPI) / FL, fl = threadIdx.x % FL;
     float x[D];
-#pragma unroll
-    for (int d = 0; d < D; ++d) x[d] = xin[i * D + d];
+    const long long row = load_point<D>(xin, order, i, x);
     constexpr int FV = F / FL; // values per lane: 1 (fp32 table) or 2 (fp16 table)
     float gy[FV];
 #pragma unroll
-    for (int f = 0; f < FV; ++f) gy[f] = (float)dLdy[i * gp.padded_width + l * F + fl * FV + f];
+    for (int f = 0; f < FV; ++f) gy[f] = live ? (float)dLdy[row * gp.padded_width + l * F + fl * FV + f] : 0.0f;
     GT *g = grad + (size_t)lv.offset[l] * F + fl * FV;
     const uint32_t size = lv.size[l], res = lv.resolution[l], flags = lv.flags[l];
     uint32_t cell[D];
     float frac[D];
     cell_of<D>(x, lv.scale[l], gp.interpolation, cell, frac);
     if (gp.interpolation == TNN_INTERP_NEAREST) {
-        if (dx == 0) add_entry<FV>(g + (size_t)level_index<D>(cell, size, res, flags, gp.hash_type) * F, gy);
+        if (dx == 0 && live) add_entry<FV>(g + (size_t)level_index<D>(cell, size, res, flags, gp.hash_type) * F, gy);
         return;
     }
 #pragma unroll
@@ -299,7 +315,32 @@ __global__ void __launch_bounds__(kGridThreads)
         float v[FV];
 #pragma unroll
         for (int f = 0; f < FV; ++f) v[f] = weight * gy[f];
-        add_entry<FV>(g + (size_t)level_index<D>(loc, size, res, flags, gp.hash_type) * F, v);
+        const uint32_t idx = level_index<D>(loc, size, res, flags, gp.hash_type);
+        if (order) {
+            // Points in cell order: neighbouring groups of lanes often hold the same entry. Runs of equal entries inside
+            // the wave are summed first (a segmented sum over the lanes LPI apart, which hold the same side and feature
+            // of the next points) and the last lane of a run adds the total: one atomic per run instead of one per point.
+            // The order of the additions is not defined in the reference either (grid.h:215-243).
+            const int wl = (int)(threadIdx.x % kGridWave);
+            const uint32_t idx_prev = (uint32_t)__shfl_up((int)idx, LPI, kGridWave);
+            bool open = wl >= LPI && idx_prev == idx; // this lane's run starts further up than the steps so far have reached
+#pragma unroll
+            for (int step = LPI; step < kGridWave; step *= 2) {
+                const bool open_up = (bool)__shfl_up((int)open, step, kGridWave);
+                float v_up[FV];
+#pragma unroll
+                for (int f = 0; f < FV; ++f) v_up[f] = __shfl_up(v[f], step, kGridWave);
+                const bool reach = wl >= step;
+#pragma unroll
+                for (int f = 0; f < FV; ++f) v[f] += (reach && open) ? v_up[f] : 0.0f;
+                open = reach ? (open && open_up) : open;
+            }
+            const uint32_t idx_down = (uint32_t)__shfl_down((int)idx, LPI, kGridWave);
+            const bool last = wl + LPI >= kGridWave || idx_down != idx;
+            if (last) add_entry<FV>(g + (size_t)idx * F, v);
+        } else {
+            add_entry<FV>(g + (size_t)idx * F, v);
+        }
     }
 }
 
@@ -353,8 +394,8 @@ static int launch_grid_forward_p(const tnn_grid_desc *d, const GridLevels &lv, c
 }
 
 template <int D, int F, typename TAB>
-static int launch_grid_backward_g(const GridLevels &lv, const GridParams &gp, const float *x, const void *dLdy, int dy_dtype,
-                                  TAB *grad, size_t M, hipStream_t s) {
+static int launch_grid_backward_g(const GridLevels &lv, const GridParams &gp, const float *x, const float4 *order, const void *dLdy,
+                                  int dy_dtype, TAB *grad, size_t M, hipStream_t s) {
     // A level goes the LDS route when its slice fits the budget and a chunk of points makes clearly more atomics
     // than the flush of the private copy does (chunk * 2^D contributions against `size` entries).
     BackwardPlan bp{};
@@ -382,7 +423,7 @@ static int launch_grid_backward_g(const GridLevels &lv, const GridParams &gp, co
         if (lds_bytes > 48 * 1024 &&                                                                                   \
             hipFuncSetAttribute(reinterpret_cast<const void *>(k), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes) != hipSuccess) \
             return fail(TNN_ERR_HIP, "cannot reserve %u bytes of LDS", lds_bytes);                                     \
-        TNN_LAUNCH(k, grid, dim3(kGridThreads), lds_bytes, s, lv, gp, bp, x, (const GT *)dLdy, grad, (long long)M);    \
+        TNN_LAUNCH(k, grid, dim3(kGridThreads), lds_bytes, s, lv, gp, bp, x, order, (const GT *)dLdy, grad, (long long)M);    \
     } while (0)
     switch (dy_dtype) {
     case TNN_FP32: TNN_BWD(float); break;
@@ -518,13 +559,14 @@ TNN_API int tnn_grid_forward_ordered(const tnn_grid_desc *desc, const void *d_or
     return rc;
 }
 
-static int grid_backward_any(const tnn_grid_desc *desc, const float *d_x, const void *d_dLdy, int dy_dtype, uint32_t padded_width,
-                             void *d_grad_table, int grad_dtype, int overwrite, size_t M, tnn_stream_t stream) {
+static int grid_backward_any(const tnn_grid_desc *desc, const float *d_x, const float4 *d_order, const void *d_dLdy, int dy_dtype,
+                             uint32_t padded_width, void *d_grad_table, int grad_dtype, int overwrite, size_t M, tnn_stream_t stream) {
     GridLevels lv;
     GridParams gp;
     int rc = grid_common(desc, padded_width, M, &lv, &gp);
     if (rc) return rc;
-    if (!d_x || !d_dLdy || !d_grad_table) return fail(TNN_ERR_INVALID_ARGUMENT, "NULL pointer argument");
+    if ((!d_x && !d_order) || !d_dLdy || !d_grad_table) return fail(TNN_ERR_INVALID_ARGUMENT, "NULL pointer argument");
+    if (d_order && (reinterpret_cast<uintptr_t>(d_order) & 15)) return fail(TNN_ERR_INVALID_ARGUMENT, "d_order must be 16-byte aligned");
     if (grad_dtype != TNN_FP32 && grad_dtype != TNN_FP16) return fail(TNN_ERR_UNSUPPORTED, "gradient table dtype %d", grad_dtype);
     if (grad_dtype == TNN_FP16 && desc->n_features_per_level % 2 != 0)
         return fail(TNN_ERR_UNSUPPORTED, "fp16 gradient tables need an even number of features per level (features are added in pairs)");
@@ -543,10 +585,10 @@ static int grid_backward_any(const tnn_grid_desc *desc, const float *d_x, const 
         if ((rc = check_launch("fill_zero_kernel"))) return rc;
     }
     if (grad_dtype == TNN_FP32) {
-        TNN_DISPATCH_DF(desc, rc = (launch_grid_backward_g<D_, F_, float>(lv, gp, d_x, d_dLdy, dy_dtype, (float *)d_grad_table, M, s)));
+        TNN_DISPATCH_DF(desc, rc = (launch_grid_backward_g<D_, F_, float>(lv, gp, d_x, d_order, d_dLdy, dy_dtype, (float *)d_grad_table, M, s)));
     } else {
         const uint32_t F = desc->n_features_per_level;
-#define TNN_PACKED(D_, F_) rc = launch_grid_backward_g<D_, F_, fp16_t>(lv, gp, d_x, d_dLdy, dy_dtype, (fp16_t *)d_grad_table, M, s)
+#define TNN_PACKED(D_, F_) rc = launch_grid_backward_g<D_, F_, fp16_t>(lv, gp, d_x, d_order, d_dLdy, dy_dtype, (fp16_t *)d_grad_table, M, s)
         if (desc->n_dims == 2) {
             if (F == 2) TNN_PACKED(2, 2); else if (F == 4) TNN_PACKED(2, 4); else TNN_PACKED(2, 8);
         } else {
@@ -559,12 +601,19 @@ static int grid_backward_any(const tnn_grid_desc *desc, const float *d_x, const 
 
 TNN_API int tnn_grid_backward(const tnn_grid_desc *desc, const float *d_x, const void *d_dLdy, int dy_dtype,
                               uint32_t padded_width, float *d_grad_table, int overwrite, size_t M, tnn_stream_t stream) {
-    return grid_backward_any(desc, d_x, d_dLdy, dy_dtype, padded_width, d_grad_table, TNN_FP32, overwrite, M, stream);
+    return grid_backward_any(desc, d_x, nullptr, d_dLdy, dy_dtype, padded_width, d_grad_table, TNN_FP32, overwrite, M, stream);
+}
+
+TNN_API int tnn_grid_backward_ordered(const tnn_grid_desc *desc, const void *d_order, const void *d_dLdy, int dy_dtype,
+                                      uint32_t padded_width, float *d_grad_table, int overwrite, size_t M, tnn_stream_t stream) {
+    if (!d_order) return tnn::fail(TNN_ERR_INVALID_ARGUMENT, "d_order is NULL");
+    return grid_backward_any(desc, nullptr, static_cast<const float4 *>(d_order), d_dLdy, dy_dtype, padded_width, d_grad_table, TNN_FP32, overwrite,
+                             M, stream);
 }
 
 TNN_API int tnn_grid_backward_packed(const tnn_grid_desc *desc, const float *d_x, const void *d_dLdy, int dy_dtype,
                                      uint32_t padded_width, void *d_grad_table_f16, int overwrite, size_t M, tnn_stream_t stream) {
-    return grid_backward_any(desc, d_x, d_dLdy, dy_dtype, padded_width, d_grad_table_f16, TNN_FP16, overwrite, M, stream);
+    return grid_backward_any(desc, d_x, nullptr, d_dLdy, dy_dtype, padded_width, d_grad_table_f16, TNN_FP16, overwrite, M, stream);
 }
 
 TNN_API int tnn_grid_indices(const tnn_grid_desc *desc, const float *d_x, uint32_t *d_indices, size_t M, tnn_stream_t stream) {

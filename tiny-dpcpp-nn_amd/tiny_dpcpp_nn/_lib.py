@@ -116,6 +116,7 @@ SIGNATURES = {
     "tnn_grid_order_points": (c_int, [POINTER(GridDesc), c_void_p, c_size_t, c_void_p, c_size_t, c_void_p]),
     "tnn_grid_forward_ordered": (c_int, [POINTER(GridDesc), c_void_p, c_void_p, c_void_p, c_int, c_uint32, c_size_t, c_void_p]),
     "tnn_grid_backward": (c_int, [POINTER(GridDesc), c_void_p, c_void_p, c_int, c_uint32, c_void_p, c_int, c_size_t, c_void_p]),
+    "tnn_grid_backward_ordered": (c_int, [POINTER(GridDesc), c_void_p, c_void_p, c_int, c_uint32, c_void_p, c_int, c_size_t, c_void_p]),
     "tnn_grid_backward_packed": (c_int, [POINTER(GridDesc), c_void_p, c_void_p, c_int, c_uint32, c_void_p, c_int, c_size_t, c_void_p]),
     "tnn_grid_indices": (c_int, [POINTER(GridDesc), c_void_p, c_void_p, c_size_t, c_void_p]),
     "tnn_grid_mlp_inference": (c_int, [POINTER(GridDesc), POINTER(MlpDesc), c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),

@@ -175,6 +175,14 @@ class Harness:
         _lib.check(self.lib.tnn_grid_backward(ctypes.byref(d), ptr(x_t), ptr(dLdy_t), dy_dtype, pw, ptr(grad_t), int(overwrite), M, self.stream()))
         return grad_t
 
+    def grid_backward_ordered(self, d, order_t, dLdy_t, dy_dtype, grad_t=None, overwrite=True):
+        M, pw = dLdy_t.shape
+        if grad_t is None:
+            grad_t = torch.full((self.grid_n_params(d),), 0.123, dtype=torch.float32, device=self.dev)
+        _lib.check(self.lib.tnn_grid_backward_ordered(ctypes.byref(d), ptr(order_t), ptr(dLdy_t), dy_dtype, pw, ptr(grad_t), int(overwrite), M,
+                                                      self.stream()))
+        return grad_t
+
     # ------------------------------------------------------------------------------
     def identity_forward(self, x_t, scale, offset, padded_width, out_dtype=FP32):
         M, D = x_t.shape

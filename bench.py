@@ -65,6 +65,8 @@ def parse():
                     help="grid_train only: gradient table in fp16 with one packed atomic per feature pair (tnn_grid_backward_packed)")
     ap.add_argument("--no-cell-order", action="store_true",
                     help="grid and grid_mlp: encode the points as they come instead of ordering the batch by cell in every step")
+    ap.add_argument("--unfused", action="store_true",
+                    help="grid_train: encoding, network step and scatter as three calls with the encoded matrix in memory")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-parity", action="store_true", help="skip the oracle check in front of the timing (profiling runs)")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -618,7 +620,33 @@ class Bench:
         order_bytes = lib.tnn_grid_order_bytes(g, M)
         order = torch.empty(max(order_bytes, 16), dtype=torch.uint8, device=t.dev)
 
+        # one call for encoding + network step + scatter (the encoded matrix never exists) unless --unfused
+        fused = not args.unfused and not args.packed_scatter
+        fws_bytes = lib.tnn_grid_mlp_train_step_workspace_bytes(g, md, M) if fused else 0
+        if fused and fws_bytes == 0:
+            raise RuntimeError(lib.tnn_last_error().decode())
+        fws = torch.empty(max(fws_bytes, 256) + 256, dtype=torch.uint8, device=t.dev)
+        fws_ptr = (fws.data_ptr() + 255) & ~255  # the workspace starts with dL/d(encoding), M x 64 of the network's type
+
+        def fused_step(i, time_scatter=False):
+            if ordered:
+                _lib.check(lib.tnn_grid_order_points(g, ptr(x), M, ptr(order), order_bytes, s))
+            _lib.check(lib.tnn_grid_mlp_train_step_l2_adam(g, md, None if ordered else ptr(x), ptr(order) if ordered else None, ptr(table), ptr(pf),
+                                                           ptr(pb), ptr(targets), loss_scale, None, ptr(loss), ptr(master), ptr(mw), ptr(vw), i + 1,
+                                                           *hyper, None, ptr(grad_table), 1, M, fws_ptr, fws_bytes, s))
+            if time_scatter:  # the scatter once more on its own, from the dL/d(encoding) the call left in its workspace
+                k0.record()
+                if ordered:
+                    _lib.check(lib.tnn_grid_backward_ordered(g, ptr(order), fws_ptr, FP16, W, ptr(grad_table), 1, M, s))
+                else:
+                    _lib.check(lib.tnn_grid_backward(g, ptr(x), fws_ptr, FP16, W, ptr(grad_table), 1, M, s))
+                k1.record()
+            _lib.check(lib.tnn_adam_step(ptr(table_master), ptr(mt), ptr(vt), ptr(grad_table), FP32, 1.0 / loss_scale, n, i + 1, *hyper,
+                                         ptr(table), FP16, s))
+
         def step(i, time_scatter=False):
+            if fused:
+                return fused_step(i, time_scatter)
             if ordered:
                 _lib.check(lib.tnn_grid_order_points(g, ptr(x), M, ptr(order), order_bytes, s))
                 _lib.check(lib.tnn_grid_forward_ordered(g, ptr(order), ptr(table), ptr(enc), FP16, W, M, s))
@@ -666,7 +694,8 @@ class Bench:
         out = line("hash-grid + fused-MLP training samples/s (2-D, 16x2, log2 19; w64, 2 hidden layers; batch 2^18; whole step with both Adam updates)",
                    "samples/s", "f16",
                    f"2-D hash-grid encoding + w64/2-hidden-layer network, one optimisation step, 2^{lg} points "
-                   f"(BASELINE config 4; gradient table {'fp16, packed atomics' if args.packed_scatter else 'fp32'})", M, tm, K, Wm, args, roof,
+                   f"(BASELINE config 4; gradient table {'fp16, packed atomics' if args.packed_scatter else 'fp32'}; "
+                   f"{'encoding inside the training kernel' if fused else 'three calls'})", M, tm, K, Wm, args, roof,
                    {"loss_first": loss0, "loss_last": float(loss.item()) * W / n_out})
         return out, cfg, w
 

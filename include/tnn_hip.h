@@ -336,6 +336,29 @@ int tnn_grid_mlp_inference(const tnn_grid_desc *grid, const tnn_mlp_desc *mlp, c
  * bit for bit. */
 int tnn_grid_mlp_inference_ordered(const tnn_grid_desc *grid, const tnn_mlp_desc *mlp, const void *d_order, const void *d_table,
                                    const void *d_prepared_fwd, void *d_y, size_t M, tnn_stream_t stream);
+
+/* One optimisation step of a network behind a hash-grid encoding without the encoded matrix (the training half of the
+ * fused path above): what the reference's training loop does with Encoding.forward, Network.forward, the L2 loss,
+ * loss.backward() through both modules and optimizer.step() on the network's parameters
+ * (dpcpp_bindings/tiny_dpcpp_nn/modules.py:357-421 over include/encodings/grid.h:661-797 and include/trainer.h:23-46).
+ * The encoding is evaluated inside the training kernel where tnn_mlp_train_step_l2_adam loads its input rows, so the
+ * M x width encoded matrix is neither written nor read; dL/d(encoding) goes through the workspace into the scatter of
+ * tnn_grid_backward (tnn_grid_backward_ordered when d_order is given). Same values as tnn_grid_forward (out_dtype = network
+ * type, padded_width = width) + tnn_mlp_train_step_l2_adam (with d_dLdx) + tnn_grid_backward: network weights and loss bit
+ * for bit, the table's gradient up to the order of its fp32 additions.
+ *   d_x: M x n_dims fp32, or NULL when d_order holds the records of tnn_grid_order_points for the batch (rows of d_targets
+ *   and d_y keep the caller's order either way). d_table: the encoding's parameters (param_dtype).
+ *   d_grad_table: n_params fp32, overwritten or accumulated into as in tnn_grid_backward; it holds loss_scale x the gradient.
+ *   Network arguments as in tnn_mlp_train_step_l2_adam. Built for width 64, ReLU, at most 4 hidden layers and 2 features per
+ *   level (tnn_grid_mlp_train_supported returns TNN_OK); other shapes get TNN_ERR_UNSUPPORTED and run the three calls.
+ * Workspace: tnn_grid_mlp_train_step_workspace_bytes. */
+int tnn_grid_mlp_train_supported(const tnn_grid_desc *grid, const tnn_mlp_desc *mlp);
+size_t tnn_grid_mlp_train_step_workspace_bytes(const tnn_grid_desc *grid, const tnn_mlp_desc *mlp, size_t M);
+int tnn_grid_mlp_train_step_l2_adam(const tnn_grid_desc *grid, const tnn_mlp_desc *mlp, const float *d_x, const void *d_order,
+                                    const void *d_table, void *d_prepared_fwd, void *d_prepared_bwd, const float *d_targets,
+                                    float loss_scale, void *d_y, float *d_loss_sum, float *d_master_packed, float *d_m, float *d_v,
+                                    int step, float lr, float beta1, float beta2, float eps, void *d_packed_T, float *d_grad_table,
+                                    int overwrite, size_t M, void *d_workspace, size_t workspace_bytes, tnn_stream_t stream);
 /* TNN_OK when tnn_grid_mlp_inference runs this pair of shapes, otherwise the status (and tnn_last_error the reason) it
  * would return: lets a caller choose between the fused call and the two calls once, when the modules are built. */
 int tnn_grid_mlp_supported(const tnn_grid_desc *grid, const tnn_mlp_desc *mlp);

@@ -122,6 +122,14 @@ SIGNATURES = {
     "tnn_grid_mlp_inference": (c_int, [POINTER(GridDesc), POINTER(MlpDesc), c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
     "tnn_grid_mlp_inference_ordered": (c_int, [POINTER(GridDesc), POINTER(MlpDesc), c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
     "tnn_grid_mlp_supported": (c_int, [POINTER(GridDesc), POINTER(MlpDesc)]),
+    "tnn_grid_mlp_train_supported": (c_int, [POINTER(GridDesc), POINTER(MlpDesc)]),
+    "tnn_grid_mlp_train_step_workspace_bytes": (c_size_t, [POINTER(GridDesc), POINTER(MlpDesc), c_size_t]),
+    "tnn_grid_mlp_train_step_l2_adam": (
+        c_int,
+        [POINTER(GridDesc), POINTER(MlpDesc), c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_void_p,
+         c_void_p, c_void_p, c_void_p, c_int, c_float, c_float, c_float, c_float, c_void_p, c_void_p, c_int, c_size_t, c_void_p, c_size_t,
+         c_void_p],
+    ),
     "tnn_identity_forward": (c_int, [c_void_p, c_uint32, c_float, c_float, c_void_p, c_int, c_uint32, c_size_t, c_void_p]),
     "tnn_frequency_forward": (c_int, [c_void_p, c_uint32, c_uint32, c_void_p, c_int, c_uint32, c_void_p, c_size_t, c_void_p]),
     "tnn_frequency_backward": (c_int, [c_void_p, c_int, c_uint32, c_void_p, c_uint32, c_uint32, c_void_p, c_size_t, c_void_p]),

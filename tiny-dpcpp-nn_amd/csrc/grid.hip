@@ -12,6 +12,7 @@
 // host and reach the kernel as scalar kernel arguments; no thread evaluates exp2.
 #include "grid_device.h"
 
+#include <algorithm>
 #include <cmath>
 #include <cstring>
 
@@ -151,10 +152,30 @@ struct BackwardPlan {
     uint32_t big_blocks;       // workgroups per other level, a group of lanes per point
     uint8_t small_level[TNN_GRID_MAX_LEVELS];
     uint8_t big_level[TNN_GRID_MAX_LEVELS];
+    // Points in cell order only: levels too large for a private copy of the whole level, where a stretch of consecutive
+    // points still lands on few enough cells for a private copy of the box around them (kMaxTiled such levels).
+    uint32_t n_tiled;
+    uint32_t budget;           // LDS bytes a workgroup may use
+    uint32_t tiled_start[17]; // first workgroup of each such level among the tiled workgroups, and their total
+    uint8_t tiled_level[16];
+    uint8_t tiled_chunk_log2[16]; // a stretch of the level is 2^n consecutive points
+    uint8_t tiled_pieces[16];     // workgroups per row of the order's coarse cells; they take the row's stretches in turn
+    uint32_t bins_per_row;        // coarse cells in a row (64 in 2-D, 16 in 3-D), n_rows rows
+    uint32_t n_rows;
 };
+constexpr uint32_t kMaxTiled = 16;
+#ifndef TNN_BOXED_MIN_PER_CELL
+#define TNN_BOXED_MIN_PER_CELL 0.3
+#endif
+constexpr double kBoxedMinPerCell = TNN_BOXED_MIN_PER_CELL; // points of the batch per cell of a level, at least, for the boxed route
 
 constexpr int kGridWave = 64;                    // lanes of a wave
-constexpr uint32_t kPrivateLdsBytes = 64 * 1024; // per workgroup; two such workgroups fit a CU
+constexpr int kBwdThreads = 512;                 // the backward kernel's workgroups
+constexpr int kDirectPasses = 8;                 // groups of kBwdThreads / lanes-per-point points a direct-route workgroup takes
+constexpr uint32_t kPrivateLdsBytes = 64 * 1024; // LDS budget of a workgroup; two such workgroups fit a CU
+// In cell order more levels take an LDS route, and the launch's LDS size holds for every workgroup, also for those of the
+// direct route, which need none: four workgroups of 40 KiB fill a CU's wave slots.
+constexpr uint32_t kPrivateLdsBytesOrdered = 40 * 1024;
 constexpr uint32_t kPrivateChunk = 4096;         // points per workgroup on the LDS route
 
 // Coordinates and row number of the i-th point: row i of x, or the i-th record of the cell order (grid_order.hip).
@@ -222,6 +243,28 @@ template <int F> __device__ __forceinline__ void add_entry(fp16_t *entry, const 
 template <int F, typename GT> struct BackwardLanes { static constexpr int FL = F; };
 template <int F> struct BackwardLanes<F, fp16_t> { static constexpr int FL = F / 2; };
 
+// Lane i of a row of 16 lanes reads lane i - N (row_shr) or i + N (row_shl) of the same row; lanes without such a
+// neighbour keep their own value.
+template <int N> __device__ __forceinline__ int row_shr(int v) {
+    if constexpr (N >= 16) return v;
+    else return __builtin_amdgcn_update_dpp(v, v, 0x110 + N, 0xf, 0xf, false);
+}
+template <int N> __device__ __forceinline__ int row_shl(int v) {
+    if constexpr (N >= 16) return v;
+    else return __builtin_amdgcn_update_dpp(v, v, 0x100 + N, 0xf, 0xf, false);
+}
+// One step of a segmented inclusive sum inside rows of 16 lanes: lanes whose run is still open take the sum STEP lanes up.
+template <int STEP, int FV> __device__ __forceinline__ void segmented_step(float (&v)[FV], bool &open, int rl) {
+    const bool open_up = row_shr<STEP>((int)open) != 0;
+    const bool reach = rl >= STEP;
+#pragma unroll
+    for (int f = 0; f < FV; ++f) {
+        const float up = __int_as_float(row_shr<STEP>(__float_as_int(v[f])));
+        v[f] += (reach && open) ? up : 0.0f;
+    }
+    open = reach ? (open && open_up) : open;
+}
+
 // Scatter-add of dL/dy into the gradient table (include/encodings/grid.h:137-245 of the reference: float atomics,
 // order not defined). Two routes inside one launch:
 //   * small levels (the coarse ones, where every point of the batch lands on a few hundred entries and global
@@ -230,21 +273,32 @@ template <int F> struct BackwardLanes<F, fp16_t> { static constexpr int FL = F /
 //   * the other levels: a group of lanes per (point, level), atomics straight to the table; workgroups of one level
 //     are dispatched together, so its slice of the table is the hot one in L2.
 template <int D, int F, typename G, typename GT>
-__global__ void __launch_bounds__(kGridThreads)
+__global__ void __launch_bounds__(kBwdThreads)
     grid_backward_kernel(const GridLevels lv, const GridParams gp, const BackwardPlan bp, const float *__restrict__ xin,
-                         const float4 *__restrict__ order, const G *__restrict__ dLdy, GT *__restrict__ grad, long long M) {
+                         const float4 *__restrict__ order, const uint32_t *__restrict__ bin_start, const G *__restrict__ dLdy,
+                         GT *__restrict__ grad, long long M) {
     extern __shared__ float priv[];
     const uint32_t n_small_blocks = bp.n_small * bp.small_blocks;
-    if (blockIdx.x < n_small_blocks) {
-        const uint32_t l = bp.small_level[blockIdx.x / bp.small_blocks];
+    // Workgroups start in the order of their numbers. Those of the LDS routes and those of the direct route are bound by
+    // different things (LDS atomics; atomic requests to memory), so their numbers are interleaved in proportion: both kinds
+    // are resident on every CU from the start, instead of one kind queueing behind the other.
+    const uint32_t n_lds_blocks = n_small_blocks + bp.tiled_start[bp.n_tiled];
+    // (Cell order only. In the caller's order the few long workgroups of the LDS route come first, as measured faster.)
+    const uint32_t n_direct_before =
+        order ? (uint32_t)(((unsigned long long)blockIdx.x * (gridDim.x - n_lds_blocks)) / gridDim.x) : (blockIdx.x < n_lds_blocks ? 0u : blockIdx.x - n_lds_blocks);
+    const bool is_direct = order ? (uint32_t)(((unsigned long long)(blockIdx.x + 1) * (gridDim.x - n_lds_blocks)) / gridDim.x) != n_direct_before
+                                 : blockIdx.x >= n_lds_blocks;
+    const uint32_t lds_block = blockIdx.x - n_direct_before; // this workgroup's number among those of its kind
+    if (!is_direct && lds_block < n_small_blocks) {
+        const uint32_t l = bp.small_level[lds_block / bp.small_blocks];
         const uint32_t size = lv.size[l], res = lv.resolution[l], flags = lv.flags[l];
         const float scale = lv.scale[l];
         const uint32_t n = size * F;
-        for (uint32_t e = threadIdx.x; e < n; e += kGridThreads) priv[e] = 0.0f;
+        for (uint32_t e = threadIdx.x; e < n; e += kBwdThreads) priv[e] = 0.0f;
         __syncthreads();
-        const long long first = (long long)(blockIdx.x % bp.small_blocks) * bp.chunk;
+        const long long first = (long long)(lds_block % bp.small_blocks) * bp.chunk;
         const long long last = first + bp.chunk < M ? first + bp.chunk : M;
-        for (long long i = first + threadIdx.x; i < last; i += kGridThreads) {
+        for (long long i = first + threadIdx.x; i < last; i += kBwdThreads) {
             float x[D];
             const long long row = load_point<D>(xin, order, i, x);
             float gy[F];
@@ -257,7 +311,7 @@ __global__ void __launch_bounds__(kGridThreads)
         }
         __syncthreads();
         GT *g = grad + (size_t)lv.offset[l] * F;
-        for (uint32_t e = threadIdx.x; e < size; e += kGridThreads) {
+        for (uint32_t e = threadIdx.x; e < size; e += kBwdThreads) {
             float v[F];
             bool any = false;
 #pragma unroll
@@ -269,17 +323,162 @@ __global__ void __launch_bounds__(kGridThreads)
         }
         return;
     }
+    if (!is_direct) {
+        // Cell order, a level whose workgroups each take stretches of consecutive points of one row of the order's coarse
+        // cells (grid_order.hip walks the coarse cells row by row, x fastest, and leaves the first position of every
+        // coarse cell behind the records): such a stretch lies in a few neighbouring cells, so the corners it touches fill
+        // a small box of the level's cells. The workgroup finds that box, accumulates in a private fp32 copy of it in LDS,
+        // and adds every touched entry to the table once. A stretch whose box does not fit (points far apart: the bins of
+        // the points outside the unit cube, a sparse region) adds to the table directly.
+        const uint32_t tb = lds_block - n_small_blocks;
+        uint32_t ti = 0;
+        while (ti + 1 < bp.n_tiled && tb >= bp.tiled_start[ti + 1]) ++ti;
+        const uint32_t l = bp.tiled_level[ti];
+        const uint32_t chunk = 1u << bp.tiled_chunk_log2[ti], pieces = bp.tiled_pieces[ti];
+        const uint32_t rowno = (tb - bp.tiled_start[ti]) / pieces, piece = (tb - bp.tiled_start[ti]) % pieces;
+        const uint32_t size = lv.size[l], res = lv.resolution[l], flags = lv.flags[l];
+        const float scale = lv.scale[l];
+        const long long row_first = bin_start[rowno * bp.bins_per_row];
+        const long long row_end = rowno + 1 < bp.n_rows ? (long long)bin_start[(rowno + 1) * bp.bins_per_row] : M;
+        __shared__ int box_lo[D], box_hi[D];
+        // lane L of wave w takes the points L * stripe + w + n_waves * k of the stretch: the lanes of an instruction are a
+        // stripe apart and rarely in the same cell, where consecutive points would queue up on one LDS address
+        constexpr uint32_t n_waves = kBwdThreads / kGridWave;
+        const uint32_t stripe = chunk / kGridWave, wv = threadIdx.x / kGridWave, ln = threadIdx.x % kGridWave;
+        const bool nearest = gp.interpolation == TNN_INTERP_NEAREST;
+        GT *g = grad + (size_t)lv.offset[l] * F;
+        for (long long first = row_first + (long long)piece * chunk; first < row_end; first += (long long)pieces * chunk) {
+            const uint32_t count = (uint32_t)((first + chunk < row_end ? first + chunk : row_end) - first);
+            __syncthreads(); // the box and the private copy of the stretch before are done with
+            if (threadIdx.x < D) {
+                box_lo[threadIdx.x] = 0x7fffffff;
+                box_hi[threadIdx.x] = (int)0x80000000;
+            }
+            __syncthreads();
+            int lo[D], hi[D];
+#pragma unroll
+            for (int d = 0; d < D; ++d) {
+                lo[d] = 0x7fffffff;
+                hi[d] = (int)0x80000000;
+            }
+            for (uint32_t k = wv; k < stripe; k += n_waves) {
+                const uint32_t pl = ln * stripe + k;
+                if (pl >= count) continue;
+                float x[D];
+                load_point<D>(xin, order, first + pl, x);
+                uint32_t cell[D];
+                float frac[D];
+                cell_of<D>(x, scale, gp.interpolation, cell, frac);
+#pragma unroll
+                for (int d = 0; d < D; ++d) {
+                    const int c = (int)cell[d];
+                    lo[d] = c < lo[d] ? c : lo[d];
+                    hi[d] = c > hi[d] ? c : hi[d];
+                }
+            }
+#pragma unroll
+            for (int d = 0; d < D; ++d) {
+#pragma unroll
+                for (int off = kGridWave / 2; off > 0; off >>= 1) {
+                    const int a = __shfl_xor(lo[d], off, kGridWave), b2 = __shfl_xor(hi[d], off, kGridWave);
+                    lo[d] = a < lo[d] ? a : lo[d];
+                    hi[d] = b2 > hi[d] ? b2 : hi[d];
+                }
+                if (ln == 0 && lo[d] <= hi[d]) {
+                    atomicMin(&box_lo[d], lo[d]);
+                    atomicMax(&box_hi[d], hi[d]);
+                }
+            }
+            __syncthreads();
+            long long n_local = 1;
+            uint32_t ext[D];
+#pragma unroll
+            for (int d = 0; d < D; ++d) {
+                lo[d] = box_lo[d];
+                const long long e = (long long)box_hi[d] - lo[d] + (nearest ? 1 : 2); // the far corners are one cell further
+                ext[d] = (uint32_t)e;
+                n_local = (e <= 0 || n_local > (1ll << 40)) ? (1ll << 41) : n_local * e;
+            }
+            const bool fits = n_local * F * (long long)sizeof(float) <= (long long)bp.budget;
+            if (fits) {
+                for (uint32_t e = threadIdx.x; e < (uint32_t)n_local * F; e += kBwdThreads) priv[e] = 0.0f;
+                __syncthreads();
+            }
+            for (uint32_t k = wv; k < stripe; k += n_waves) {
+                const uint32_t pl = ln * stripe + k;
+                if (pl >= count) continue;
+                float x[D];
+                const long long row = load_point<D>(xin, order, first + pl, x);
+                float gy[F];
+#pragma unroll
+                for (int f = 0; f < F; ++f) gy[f] = (float)dLdy[row * gp.padded_width + l * F + f];
+                uint32_t cell[D];
+                float frac[D];
+                cell_of<D>(x, scale, gp.interpolation, cell, frac);
+#pragma unroll
+                for (int c = 0; c < (1 << D); ++c) {
+                    if (nearest && c > 0) break;
+                    float weight = 1.0f;
+                    uint32_t loc[D];
+                    uint32_t local = 0, stride = 1;
+#pragma unroll
+                    for (int d = 0; d < D; ++d) {
+                        const bool far = !nearest && (c & (1 << d));
+                        weight *= nearest ? 1.0f : (far ? frac[d] : 1 - frac[d]); // the products of for_each_corner
+                        loc[d] = far ? cell[d] + 1 : cell[d];
+                        local += (uint32_t)((int)loc[d] - lo[d]) * stride;
+                        stride *= ext[d];
+                    }
+                    if (fits) {
+#pragma unroll
+                        for (int f = 0; f < F; ++f) atomicAdd(&priv[local * F + f], weight * gy[f]);
+                    } else {
+                        float v[F];
+#pragma unroll
+                        for (int f = 0; f < F; ++f) v[f] = weight * gy[f];
+                        add_entry<F>(g + (size_t)level_index<D>(loc, size, res, flags, gp.hash_type) * F, v);
+                    }
+                }
+            }
+            if (!fits) continue;
+            __syncthreads();
+            for (uint32_t e = threadIdx.x; e < (uint32_t)n_local; e += kBwdThreads) {
+                float v[F];
+                bool any = false;
+#pragma unroll
+                for (int f = 0; f < F; ++f) {
+                    v[f] = priv[e * F + f];
+                    any |= v[f] != 0.0f;
+                }
+                if (!any) continue;
+                uint32_t loc[D], rest = e;
+#pragma unroll
+                for (int d = 0; d < D; ++d) {
+                    loc[d] = (uint32_t)(lo[d] + (int)(rest % ext[d]));
+                    rest /= ext[d];
+                }
+                add_entry<F>(g + (size_t)level_index<D>(loc, size, res, flags, gp.hash_type) * F, v);
+            }
+        }
+        return;
+    }
     // A group of 2 * FL neighbouring lanes owns one (point, level): lane (dx, fl) adds feature fl (fp16 table: the pair of
     // features fl) of the corners on side dx of the cell along the first dimension. The memory side retires atomic
     // requests per 32-byte sector, about 20 * 10^9 a second, however many lanes of one instruction fall into the sector:
     // the features of an entry always do, and the two corners along the first dimension are neighbouring entries
     // wherever that dimension enters the index unhashed or the hash leaves it in the low bits.
     constexpr int FL = BackwardLanes<F, GT>::FL, LPI = 2 * FL;
-    const uint32_t b = blockIdx.x - n_small_blocks;
+    const uint32_t b = n_direct_before;
     const uint32_t l = bp.big_level[b / bp.big_blocks];
-    const long long i_raw = (long long)(b % bp.big_blocks) * (kGridThreads / LPI) + threadIdx.x / LPI;
+    // kDirectPasses groups of points per workgroup, one after the other: a workgroup that ended after two atomics per lane
+    // left the launch bound by the rate at which workgroups are dispatched
+    GT *const g = grad + (size_t)lv.offset[l] * F + (threadIdx.x % FL) * (F / FL);
+    const uint32_t size = lv.size[l], res = lv.resolution[l], flags = lv.flags[l];
+    for (int pass = 0; pass < kDirectPasses; ++pass) {
+    const long long i_raw = ((long long)(b % bp.big_blocks) * kDirectPasses + pass) * (kBwdThreads / LPI) + threadIdx.x / LPI;
     const bool live = i_raw < M;
-    if (!live && !order) return;
+    if (i_raw - threadIdx.x / LPI >= M) break; // the whole workgroup is past the end
+    if (!live && !order) continue;
     const long long i = live ? i_raw : M - 1; // in cell order every lane stays for the exchange between lanes below
     const int dx = (threadIdx.x % LPI) / FL, fl = threadIdx.x % FL;
     float x[D];
@@ -288,14 +487,12 @@ __global__ void __launch_bounds__(kGridThreads)
     float gy[FV];
 #pragma unroll
     for (int f = 0; f < FV; ++f) gy[f] = live ? (float)dLdy[row * gp.padded_width + l * F + fl * FV + f] : 0.0f;
-    GT *g = grad + (size_t)lv.offset[l] * F + fl * FV;
-    const uint32_t size = lv.size[l], res = lv.resolution[l], flags = lv.flags[l];
     uint32_t cell[D];
     float frac[D];
     cell_of<D>(x, lv.scale[l], gp.interpolation, cell, frac);
     if (gp.interpolation == TNN_INTERP_NEAREST) {
         if (dx == 0 && live) add_entry<FV>(g + (size_t)level_index<D>(cell, size, res, flags, gp.hash_type) * F, gy);
-        return;
+        continue;
     }
 #pragma unroll
     for (int rest = 0; rest < (1 << (D - 1)); ++rest) {
@@ -317,30 +514,28 @@ __global__ void __launch_bounds__(kGridThreads)
         for (int f = 0; f < FV; ++f) v[f] = weight * gy[f];
         const uint32_t idx = level_index<D>(loc, size, res, flags, gp.hash_type);
         if (order) {
-            // Points in cell order: neighbouring groups of lanes often hold the same entry. Runs of equal entries inside
-            // the wave are summed first (a segmented sum over the lanes LPI apart, which hold the same side and feature
+            // Points in cell order: neighbouring groups of lanes often hold the same entry. Runs of equal entries inside a row
+            // of 16 lanes are summed first (a segmented sum over the lanes LPI apart, which hold the same side and feature
             // of the next points) and the last lane of a run adds the total: one atomic per run instead of one per point.
-            // The order of the additions is not defined in the reference either (grid.h:215-243).
-            const int wl = (int)(threadIdx.x % kGridWave);
-            const uint32_t idx_prev = (uint32_t)__shfl_up((int)idx, LPI, kGridWave);
-            bool open = wl >= LPI && idx_prev == idx; // this lane's run starts further up than the steps so far have reached
-#pragma unroll
-            for (int step = LPI; step < kGridWave; step *= 2) {
-                const bool open_up = (bool)__shfl_up((int)open, step, kGridWave);
-                float v_up[FV];
-#pragma unroll
-                for (int f = 0; f < FV; ++f) v_up[f] = __shfl_up(v[f], step, kGridWave);
-                const bool reach = wl >= step;
-#pragma unroll
-                for (int f = 0; f < FV; ++f) v[f] += (reach && open) ? v_up[f] : 0.0f;
-                open = reach ? (open && open_up) : open;
+            // Lanes exchange through DPP row shifts, not through the LDS crossbar, which the workgroups of the LDS routes
+            // on the same CU keep busy with their atomics. The order of the additions is not defined in the reference
+            // either (grid.h:215-243).
+            const int rl = (int)(threadIdx.x % 16);
+            const uint32_t idx_prev = (uint32_t)row_shr<LPI>((int)idx);
+            bool open = rl >= LPI && idx_prev == idx; // this lane's run starts further up than the steps so far have reached
+            if constexpr (LPI < 16) {
+                segmented_step<LPI, FV>(v, open, rl);
+                if constexpr (2 * LPI < 16) segmented_step<2 * LPI, FV>(v, open, rl);
+                if constexpr (4 * LPI < 16) segmented_step<4 * LPI, FV>(v, open, rl);
+                if constexpr (8 * LPI < 16) segmented_step<8 * LPI, FV>(v, open, rl);
             }
-            const uint32_t idx_down = (uint32_t)__shfl_down((int)idx, LPI, kGridWave);
-            const bool last = wl + LPI >= kGridWave || idx_down != idx;
+            const uint32_t idx_next = (uint32_t)row_shl<LPI>((int)idx);
+            const bool last = rl + LPI >= 16 || idx_next != idx;
             if (last) add_entry<FV>(g + (size_t)idx * F, v);
         } else {
             add_entry<FV>(g + (size_t)idx * F, v);
         }
+    }
     }
 }
 
@@ -400,21 +595,62 @@ static int launch_grid_backward_g(const GridLevels &lv, const GridParams &gp, co
     // than the flush of the private copy does (chunk * 2^D contributions against `size` entries).
     BackwardPlan bp{};
     bp.chunk = kPrivateChunk;
+    bp.budget = order ? kPrivateLdsBytesOrdered : kPrivateLdsBytes;
     bp.small_blocks = (uint32_t)((M + bp.chunk - 1) / bp.chunk);
-    constexpr int per_block = kGridThreads / (2 * BackwardLanes<F, TAB>::FL); // (point, level) pairs per workgroup on the direct route
+    constexpr int per_block = kDirectPasses * kBwdThreads / (2 * BackwardLanes<F, TAB>::FL); // (point, level) pairs per workgroup on the direct route
     bp.big_blocks = (uint32_t)((M + per_block - 1) / per_block);
     const size_t per_chunk = (M < bp.chunk ? M : (size_t)bp.chunk) << (gp.interpolation == TNN_INTERP_NEAREST ? 0 : D);
     uint32_t n_big = 0, lds_bytes = 0;
     for (uint32_t l = 0; l < gp.n_levels; ++l) {
         const size_t bytes = (size_t)lv.size[l] * F * sizeof(float);
-        if (bytes <= kPrivateLdsBytes && per_chunk >= 2 * (size_t)lv.size[l]) {
+        // (in cell order only the coarsest levels: the box of a stretch is far smaller than a level from 8 KiB on)
+        if (bytes <= (order ? 8192u : bp.budget) && per_chunk >= 2 * (size_t)lv.size[l]) {
             bp.small_level[bp.n_small++] = (uint8_t)l;
             if (bytes > lds_bytes) lds_bytes = (uint32_t)bytes;
         } else {
             bp.big_level[n_big++] = (uint8_t)l;
         }
     }
-    const unsigned long long blocks = (unsigned long long)bp.n_small * bp.small_blocks + (unsigned long long)n_big * bp.big_blocks;
+    // Cell order: of the other levels, those where a stretch of consecutive points of one row of the order's coarse cells
+    // fills a box of the level's cells that fits the LDS budget take the boxed route, as long as the level has a point for
+    // every few cells (beyond that a box holds hardly more than one contribution per entry and saves no atomics). The order
+    // (grid_order.hip) walks a lattice of 64^2 (16^3) coarse cells row by row, x fastest: with the points spread evenly a
+    // row holds M / 64 (M / 256) of them, and a stretch of C of these spans that share of the level's width plus a coarse
+    // cell, and one coarse cell in the other dimensions. A stretch that breaks the estimate is caught in the kernel.
+    const uint32_t *bin_start = nullptr;
+    if (order && gp.n_levels > 0 && gp.interpolation != TNN_INTERP_NEAREST) {
+        bin_start = reinterpret_cast<const uint32_t *>(reinterpret_cast<const char *>(order) + order_record_bytes(M));
+        bp.bins_per_row = (D == 2) ? 64 : 16;
+        bp.n_rows = 4096 / bp.bins_per_row;
+        const double per_row = (double)M / bp.n_rows, coarse = (double)bp.bins_per_row;
+        uint32_t kept = 0;
+        for (uint32_t i = 0; i < n_big; ++i) {
+            const uint32_t l = bp.big_level[i];
+            const double R = (double)lv.resolution[l];
+            const double per_cell = (double)M / std::pow(R, (double)D);
+            int chunk_log2 = -1;
+            // (short stretches: many workgroups of some ten microseconds each spread over the CUs far more evenly than few long ones)
+            for (int c = 10; c >= 9 && chunk_log2 < 0 && bp.n_tiled < kMaxTiled && per_cell >= kBoxedMinPerCell; --c) {
+                const double share = std::min(1.0, (double)(1u << c) / std::max(per_row, 1.0));
+                double cells = (share * R + R / coarse + 2.0) * (R / coarse + 2.0);
+                if (D == 3) cells *= R / coarse + 2.0;
+                if (cells * F * sizeof(float) <= 0.9 * (double)bp.budget) chunk_log2 = c;
+            }
+            if (chunk_log2 >= 0) {
+                const uint32_t pieces = (uint32_t)std::min(64.0, std::ceil(per_row / (double)(1u << chunk_log2)) + 1.0);
+                bp.tiled_level[bp.n_tiled] = (uint8_t)l;
+                bp.tiled_chunk_log2[bp.n_tiled] = (uint8_t)chunk_log2;
+                bp.tiled_pieces[bp.n_tiled] = (uint8_t)pieces;
+                bp.tiled_start[bp.n_tiled + 1] = bp.tiled_start[bp.n_tiled] + bp.n_rows * pieces;
+                ++bp.n_tiled;
+                if (bp.budget > lds_bytes) lds_bytes = bp.budget;
+            } else {
+                bp.big_level[kept++] = (uint8_t)l;
+            }
+        }
+        n_big = kept;
+    }
+    const unsigned long long blocks = (unsigned long long)bp.n_small * bp.small_blocks + bp.tiled_start[bp.n_tiled] + (unsigned long long)n_big * bp.big_blocks;
     if (blocks > 0x7fffffffull) return fail(TNN_ERR_UNSUPPORTED, "grid backward: batch too large for one launch");
     const dim3 grid((unsigned)blocks);
 #define TNN_BWD(GT)                                                                                                    \
@@ -423,7 +659,7 @@ static int launch_grid_backward_g(const GridLevels &lv, const GridParams &gp, co
         if (lds_bytes > 48 * 1024 &&                                                                                   \
             hipFuncSetAttribute(reinterpret_cast<const void *>(k), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes) != hipSuccess) \
             return fail(TNN_ERR_HIP, "cannot reserve %u bytes of LDS", lds_bytes);                                     \
-        TNN_LAUNCH(k, grid, dim3(kGridThreads), lds_bytes, s, lv, gp, bp, x, order, (const GT *)dLdy, grad, (long long)M);    \
+        TNN_LAUNCH(k, grid, dim3(kBwdThreads), lds_bytes, s, lv, gp, bp, x, order, bin_start, (const GT *)dLdy, grad, (long long)M);    \
     } while (0)
     switch (dy_dtype) {
     case TNN_FP32: TNN_BWD(float); break;

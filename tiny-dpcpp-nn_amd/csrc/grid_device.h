@@ -27,6 +27,10 @@ struct GridParams {
     uint32_t padded_width;
 };
 
+// The buffer of tnn_grid_order_points (grid_order.hip): M records of 16 bytes, padded to 256 bytes, then the first position
+// of each of the 4096 coarse cells of the order (uint32, key order), which the scatter over ordered points reads.
+inline size_t order_record_bytes(size_t M) { return (M * 16 + 255) & ~(size_t)255; }
+
 // Host side (grid.hip): validation of a descriptor, and of a call (include/encodings/grid.h:665-677) together with
 // the per-level constants the kernels take.
 int check_grid_desc(const tnn_grid_desc *d);

@@ -38,7 +38,7 @@ static OrderPlan order_plan(size_t M) {
     p.n_wg = (int)wg;
     long long chunk = ((long long)M + wg - 1) / wg;
     p.chunk = (chunk + kOrderThreads - 1) / kOrderThreads * kOrderThreads;
-    p.record_bytes = (M * 16 + 255) & ~(size_t)255;
+    p.record_bytes = order_record_bytes(M);
     p.hist_bytes = (size_t)p.n_wg * kOrderBins * sizeof(uint32_t);
     p.group_bytes = (size_t)p.n_wg * kOrderGroups * sizeof(uint32_t);
     return p;

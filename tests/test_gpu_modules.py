@@ -464,6 +464,31 @@ def test_large_batches_take_the_cell_order_route(tcnn):
     assert float(big.float().abs().max()) > 1e-3
 
 
+def test_large_batches_scatter_in_cell_order(tcnn):
+    """From 2^17 rows on the grid encoding's backward pass orders the batch by cell and scatters over the ordered points. The
+    gradient of the table is a sum over rows: the large batch's gradient equals the sum of the gradients of its two halves
+    (each below the threshold, scattered in the caller's order) up to fp32 rounding of sums in another order."""
+    n = 1 << 17
+    cfg = {"otype": "HashGrid", "n_levels": 16, "n_features_per_level": 2, "log2_hashmap_size": 15, "base_resolution": 16, "per_level_scale": 1.5}
+    torch.manual_seed(6)
+    enc = tcnn.Encoding(2, cfg, dtype=torch.float32)
+    with torch.no_grad():
+        enc.params.copy_(torch.rand_like(enc.params) * 2 - 1)
+    x = torch.rand((n, 2), device=DEVICE)
+    w = torch.randn((n, enc.n_output_dims), device=DEVICE)
+
+    def grad_of(rows):
+        enc.params.grad = None
+        (enc(x[rows]).float() * w[rows]).sum().backward()
+        return enc.params.grad.clone()
+
+    whole = grad_of(slice(0, n))
+    halves = grad_of(slice(0, n // 2)) + grad_of(slice(n // 2, n))
+    scale = float(halves.abs().max())
+    assert scale > 1.0
+    assert float((whole - halves).abs().max()) <= 2e-5 * scale
+
+
 def test_nerf_style_directional_network(tcnn):
     """test/python/test_nerf_settings.py:80-86 of the reference: spherical harmonics of degree 4 feeding a network."""
     model = tcnn.NetworkWithInputEncoding(3, 3, net_config(64, 2), {"otype": "SphericalHarmonics", "degree": 4}, dtype=torch.bfloat16)

@@ -40,14 +40,15 @@ METRIC = "fused-MLP train & infer samples/s (w64, batch 2^18); % bf16 MFMA peak"
 # x2.000 and x1.000). The summaries with the commands are profiles/mlp_train_fused_kernel.*.txt, profiles/mlp_forward_kernel.*.txt,
 # profiles/grid_forward_kernel.*.txt, profiles/grid_mlp_inference_kernel.*.txt and profiles/grid_backward_kernel.*.txt. Not measured live: counters need the profiler.
 MEASURED_TRAFFIC_BYTES = {
-    ("train", 18): (56840.5 * 2.0 + 20488.0) * 1024,
+    ("train", 18): (55832.3 * 2.0 + 20488.0) * 1024,
     ("infer", 18): (16786.6 * 2.0 + 32768.0) * 1024,
     ("train_fb", 18): (98600.2 * 2.0 + 217143.4) * 1024,  # the backward kernel
     ("grid", 21): (6374561.8 * 2.0 + 132047.2) * 1024,           # points in the caller's order (--no-cell-order)
     ("grid_ordered", 21): (3584394.4 * 2.0 + 131865.3) * 1024,   # points in cell order, the default
     ("grid_mlp", 21): (6610053.5 * 2.0 + 263715.5) * 1024,
     ("grid_mlp_ordered", 21): (3915783.4 * 2.0 + 264728.9) * 1024,
-    ("grid_train", 18): (211580.8 * 2.0 + 236762.7) * 1024,  # the scatter kernel; an atomic request counts as a 32-byte write
+    ("grid_train", 18): (108943.2 * 2.0 + 236762.7) * 1024,  # the scatter kernel; an atomic request counts as a 32-byte write
+    ("grid_train_ordered", 18): (248862.1 * 2.0 + 126583.5) * 1024,
 }
 
 
@@ -687,7 +688,7 @@ class Bench:
         lg = int(np.log2(M))
         ach = bpp * M / (scatter_ms * 1e-3) / 1e9
         roof = {"bound": "hbm", "achieved": ach, "peak": PEAK_HBM, "unit": "GB/s", "frac": ach / PEAK_HBM,
-                "traffic": MEASURED_TRAFFIC_BYTES.get(("grid_train_packed" if args.packed_scatter else "grid_train", lg)),
+                "traffic": MEASURED_TRAFFIC_BYTES.get(("grid_train_packed" if args.packed_scatter else ("grid_train_ordered" if ordered else "grid_train"), lg)),
                 "kernel": "grid_backward_kernel (with the fill of the gradient table in front of it)" + (" over points in cell order" if ordered else ""),
                 "kernel_ms": scatter_ms,
                 "algorithmic_bytes_per_launch": bpp * M}

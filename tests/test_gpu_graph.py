@@ -76,3 +76,75 @@ def test_captured_step_replays_like_eager(tnn):
                 assert torch.allclose(a, b, rtol=1e-4, atol=1e-6 * float(a.abs().max())), f"replay {it}: {name}"
             else:
                 assert torch.equal(a, b), f"replay {it}: {name}"
+
+
+def test_captured_fused_grid_step_replays_like_eager(tnn):
+    """The same for the step that orders the batch by cell and runs encoding, network step (with Adam) and scatter as one call:
+    tnn_grid_order_points + tnn_grid_mlp_train_step_l2_adam recorded once, replayed on new points and targets. The weights are
+    restored before every run so that eager and replayed steps start from the same state."""
+    M, n_hidden = 1 << 14, 2
+    n_mats = n_hidden + 1
+    gen = torch.Generator(device=tnn.dev).manual_seed(10)
+    gd = tnn.grid_desc(CFG, FP16)
+    g = ctypes.byref(gd)
+    n_table = tnn.grid_n_params(gd)
+    table = (torch.rand(n_table, device=tnn.dev, generator=gen) * 2 - 1).to(torch.float16)
+    desc = tnn.mlp_desc(FP16, W, n_hidden, "relu", "none")
+    d = ctypes.byref(desc)
+    master0 = (torch.rand(n_mats * W * W, device=tnn.dev, generator=gen) * 2 - 1) * 0.2
+    master = master0.clone()
+    pf0, pb0 = tnn.prepare_packed(desc, master0, src_is_fp32=True)
+    pf, pb = pf0.clone(), pb0.clone()
+    m, v = torch.zeros_like(master), torch.zeros_like(master)
+    x = torch.rand((M, 2), device=tnn.dev, generator=gen)
+    targets = torch.rand((M, W), device=tnn.dev, generator=gen)
+    y = torch.empty((M, W), dtype=torch.float16, device=tnn.dev)
+    loss = torch.zeros(1, device=tnn.dev)
+    grad_table = torch.empty(n_table, device=tnn.dev)
+    order_bytes = tnn.lib.tnn_grid_order_bytes(g, M)
+    order = torch.empty(order_bytes, dtype=torch.uint8, device=tnn.dev)
+    ws_bytes = tnn.lib.tnn_grid_mlp_train_step_workspace_bytes(g, d, M)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=tnn.dev)
+
+    def restore():
+        master.copy_(master0); pf.copy_(pf0); pb.copy_(pb0); m.zero_(); v.zero_()
+
+    def step():
+        s = tnn.stream()
+        _lib.check(tnn.lib.tnn_grid_order_points(g, ptr(x), M, ptr(order), order_bytes, s))
+        _lib.check(tnn.lib.tnn_grid_mlp_train_step_l2_adam(g, d, None, ptr(order), ptr(table), ptr(pf), ptr(pb), ptr(targets), 4096.0, ptr(y),
+                                                           ptr(loss), ptr(master), ptr(m), ptr(v), 1, 1e-2, 0.9, 0.99, 1e-8, None, ptr(grad_table), 1,
+                                                           M, ptr(ws), ws_bytes, s))
+
+    def snapshot():
+        torch.cuda.synchronize()
+        return [t.clone() for t in (y, loss, master, pf, pb, grad_table)]
+
+    step()
+    torch.cuda.synchronize()
+    restore()
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            step()
+    torch.cuda.current_stream().wait_stream(side)
+
+    for it in range(4):
+        x.copy_(torch.rand((M, 2), device=tnn.dev, generator=gen))
+        targets.copy_(torch.rand((M, W), device=tnn.dev, generator=gen))
+        restore()
+        step()
+        eager = snapshot()
+        restore()
+        for t in (y, loss, grad_table):
+            t.fill_(float("nan"))
+        graph.replay()
+        replayed = snapshot()
+        for name, a, b in zip(("y", "loss", "master", "forward weights", "backward weights", "gradient table"), eager, replayed):
+            if name == "gradient table":
+                assert torch.allclose(a, b, rtol=1e-4, atol=1e-6 * float(a.abs().max())), f"replay {it}: {name}"
+            else:
+                assert torch.equal(a, b), f"replay {it}: {name}"
+        assert float(eager[1]) > 0

@@ -120,7 +120,8 @@ def test_config_5_full_size_ordered(tnn, oracle):
 @pytest.mark.parametrize("cfg,pd", [(CFG4, FP16), (CFG5, FP16), (dict(CFG5, n_features_per_level=4, n_levels=8, interpolation="Smoothstep"), FP32),
                                     (dict(CFG4, grid_type="Dense", n_levels=6, n_features_per_level=1), FP16),
                                     (dict(CFG5, hash="Prime", n_features_per_level=8, n_levels=4, interpolation="Nearest"), FP16)])
-@pytest.mark.parametrize("kind,M", [("uniform", 2011), ("uniform", 70000), ("clustered", 30001), ("identical", 777), ("uniform", 1)])
+@pytest.mark.parametrize("kind,M", [("uniform", 2011), ("uniform", 70000), ("clustered", 30001), ("identical", 777), ("uniform", 1),
+                                    ("wild", 9001)])
 def test_ordered_backward_matches_the_oracle(tnn, oracle, cfg, pd, kind, M):
     """tnn_grid_backward_ordered: the same contributions as tnn_grid_backward, summed per run of equal entries inside a wave
     first. fp32 sums in another order against the oracle's double sum: |err| <= 1e-5 x the largest entry (the bar of the
@@ -128,6 +129,8 @@ def test_ordered_backward_matches_the_oracle(tnn, oracle, cfg, pd, kind, M):
     D, F, L = cfg["n_dims"], cfg["n_features_per_level"], cfg["n_levels"]
     rng = np.random.default_rng(M + 31 * D + F)
     x = points(kind, M, D, rng)
+    if kind == "wild":  # points outside the unit cube: bins whose boxes do not fit (a NaN coordinate has no defined cell)
+        x = np.nan_to_num(x, nan=0.25, posinf=1.5, neginf=-0.5)
     pw = L * F + 8
     d = tnn.grid_desc(cfg, pd)
     n = tnn.grid_n_params(d)
@@ -157,3 +160,21 @@ def test_ordered_backward_config_4_full_size(tnn, oracle):
     ref = oracle.grid_backward(cfg, x.cpu().numpy(), g.to(torch.float32).cpu().numpy(), n)
     assert np.abs(grad - ref).max() <= 1e-5 * np.abs(ref).max() + 1e-4
     assert_close(grad, ref, FP32, "gradient table", scale=1e2, frac_ok=1e-4)
+
+
+@pytest.mark.parametrize("cfg,M", [(CFG4, (1 << 20) + 8), (dict(CFG5, log2_hashmap_size=19), 1 << 20), (dict(CFG4, base_resolution=4, n_levels=12), 1 << 16)])
+def test_ordered_backward_plans_at_other_sizes(tnn, cfg, M):
+    """Batch sizes and level sets that change which levels take which route (stretch length, workgroups per coarse row, 3-D
+    boxes): the ordered scatter against the plain one, both fp32 atomics: |a - b| <= 2e-5 x the largest entry."""
+    d = tnn.grid_desc(cfg, FP16)
+    gen = torch.Generator(device=tnn.dev).manual_seed(M % 1000)
+    x = torch.rand((M, cfg["n_dims"]), device=tnn.dev, generator=gen)
+    x[: M // 4] = x[: M // 4] * 0.05 + 0.4   # a quarter of the points in a small region: long coarse rows
+    pw = cfg["n_levels"] * cfg["n_features_per_level"]
+    g = (torch.rand((M, pw), device=tnn.dev, generator=gen) - 0.5).to(torch.float16)
+    plain = tnn.grid_backward(d, x, g, FP16)
+    ordered = tnn.grid_backward_ordered(d, tnn.grid_order(d, x), g, FP16)
+    tnn.sync()
+    scale = float(plain.abs().max())
+    assert scale > 0
+    assert float((plain - ordered).abs().max()) <= 2e-5 * scale

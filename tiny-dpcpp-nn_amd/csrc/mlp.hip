@@ -13,6 +13,7 @@
 // the fp32 accumulator before rounding).
 #include "mlp_tile.h"
 #include "mlp_train_shape.h"
+#include "mlp_backward128.inc"
 
 #include <cstdlib>
 
@@ -792,6 +793,62 @@ static int launch_dw(const tnn_mlp_desc *d, const void *interm_bwd, const void *
     return check_launch("dw_reduce_kernel");
 }
 
+// Width 128: one launch per layer that forms delta_{l-1} and dW_l together (mlp_backward128.inc), then the reduction.
+// With `targets` the top layer's launch forms dL/dy itself from the network's output (the last matrix of interm_fwd) and adds
+// the loss values into *loss_sum (zeroed by the caller); dLdy is then not read.
+template <typename T>
+static int launch_backward128(const tnn_mlp_desc *d, const void *wprep_bwd, const void *dLdy, const void *interm_fwd, void *deltas,
+                              bool keep_top_delta, void *dW, int dW_is_fp32, void *dLdx, size_t M, float *partials, hipStream_t s,
+                              const float *targets = nullptr, float loss_scale = 0.0f, float *loss_sum = nullptr) {
+    typedef typename Storage<T>::vec8 vec8;
+    constexpr int W = 128;
+    const int n_mats = d->n_hidden_layers + 1;
+    const DwPlan p = dw_plan(d, M);
+    const size_t mat = M * W, per_mat = (size_t)4 * 8 * 64;
+    auto k_top = targets ? mlp_layer_backward128_kernel<T, 2> : mlp_layer_backward128_kernel<T, 1>;
+    auto k_mid = mlp_layer_backward128_kernel<T, 0>;
+    const float inv_n = 1.0f / (float)(M * W);
+    for (auto k : {k_top, k_mid})
+        if (hipFuncSetAttribute(reinterpret_cast<const void *>(k), hipFuncAttributeMaxDynamicSharedMemorySize, (int)LayerBwd128::lds_bytes) != hipSuccess)
+            return fail(TNN_ERR_HIP, "cannot reserve %zu bytes of LDS", LayerBwd128::lds_bytes);
+    const T *fwd = static_cast<const T *>(interm_fwd);
+    T *dl = static_cast<T *>(deltas);
+    for (int l = n_mats - 1; l >= 0; --l) {
+        const bool top = (l == n_mats - 1);
+        const T *delta_in = top ? static_cast<const T *>(dLdy) : dl + (size_t)l * mat;
+        T *delta_out = l > 0 ? dl + (size_t)(l - 1) * mat : static_cast<T *>(dLdx);
+        const int gate = l > 0 ? d->activation : TNN_ACT_NONE;
+        TNN_LAUNCH((top ? k_top : k_mid), dim3((unsigned)p.n_chunks), dim3(kLayerBwdThreads), LayerBwd128::lds_bytes, s,
+                   (const vec8 *)wprep_bwd + (size_t)l * per_mat, delta_in, fwd + (size_t)l * mat, fwd + (size_t)n_mats * mat,
+                   (top && keep_top_delta) ? dl + (size_t)l * mat : (T *)nullptr, delta_out, partials, n_mats, l, gate, d->output_activation,
+                   (long long)M, p.rows_per_chunk, targets, loss_scale, inv_n, loss_sum);
+        const int rc = check_launch("mlp_layer_backward128_kernel");
+        if (rc) return rc;
+    }
+    const int n_elems = n_mats * W * W;
+    TNN_LAUNCH((dw_reduce_kernel<T>), dim3(n_elems / 64), dim3(512), 0, s, partials, (int)(p.n_chunks * p.partials_per_chunk), n_elems,
+               dW_is_fp32 ? (T *)nullptr : (T *)dW, dW_is_fp32 ? (float *)dW : (float *)nullptr);
+    return check_launch("dw_reduce_kernel");
+}
+
+// For tnn_mlp_train_step_l2 on width 128: loss and backward pass over stored activations, the loss folded into the top
+// layer's launch. Workspace as tnn_mlp_backward's.
+int backward128_from_loss(const tnn_mlp_desc *desc, const void *wprep_bwd, const void *interm_fwd, const float *targets, float loss_scale,
+                          float *loss_sum, void *dW, int dW_is_fp32, void *dLdx, size_t M, void *workspace, size_t workspace_bytes, hipStream_t s) {
+    const DwPlan p = dw_plan(desc, M);
+    const size_t partial_rounded = (p.partial_bytes + 255) & ~(size_t)255;
+    const size_t need = partial_rounded + p.delta_bytes + 512;
+    if (!workspace || workspace_bytes < need) return fail(TNN_ERR_WORKSPACE, "workspace of %zu bytes given, %zu needed", workspace_bytes, need);
+    uintptr_t base = (reinterpret_cast<uintptr_t>(workspace) + 255) & ~(uintptr_t)255;
+    float *partials = reinterpret_cast<float *>(base);
+    void *deltas = reinterpret_cast<void *>(base + partial_rounded);
+    if (desc->dtype == TNN_BF16)
+        return launch_backward128<bf16_t>(desc, wprep_bwd, nullptr, interm_fwd, deltas, false, dW, dW_is_fp32, dLdx, M, partials, s, targets, loss_scale,
+                                          loss_sum);
+    return launch_backward128<fp16_t>(desc, wprep_bwd, nullptr, interm_fwd, deltas, false, dW, dW_is_fp32, dLdx, M, partials, s, targets, loss_scale,
+                                      loss_sum);
+}
+
 #define TNN_DISPATCH_TW(desc, CALL)                                                          \
     do {                                                                                     \
         if ((desc)->dtype == TNN_BF16) {                                                     \
@@ -902,6 +959,13 @@ TNN_API int tnn_mlp_backward(const tnn_mlp_desc *desc, const void *d_prepared_bw
     // then written only if the caller asked for them
     rc = fused_backward(desc, d_prepared_bwd, d_dLdy, d_interm_fwd, d_interm_bwd, d_dW, dW_is_fp32, d_dLdx, M, partials, p.partial_bytes, s);
     if (rc != TNN_ERR_UNSUPPORTED) return rc;
+    if (desc->width == 128) {
+        if (desc->dtype == TNN_BF16)
+            return launch_backward128<bf16_t>(desc, d_prepared_bwd, d_dLdy, d_interm_fwd, deltas, d_interm_bwd != nullptr, d_dW, dW_is_fp32, d_dLdx, M,
+                                              partials, s);
+        return launch_backward128<fp16_t>(desc, d_prepared_bwd, d_dLdy, d_interm_fwd, deltas, d_interm_bwd != nullptr, d_dW, dW_is_fp32, d_dLdx, M,
+                                          partials, s);
+    }
     TNN_DISPATCH_TW(desc, rc = (launch_backward<T_, W_>(desc, d_prepared_bwd, d_dLdy, d_interm_fwd, deltas, d_dLdx, M, s)));
     if (rc) return rc;
     TNN_DISPATCH_TW(desc, rc = (launch_dw<T_, W_>(desc, deltas, d_interm_fwd, d_dW, dW_is_fp32, M, partials, s)));

@@ -38,6 +38,9 @@ int fused_train_step(const tnn_mlp_desc *d, const void *wf, const void *wb, cons
                      void *y, float *loss_sum, void *dW, int dW_is_fp32, void *dx, size_t M, void *ws, size_t ws_bytes, const TrainTail &tail,
                      hipStream_t s);
 size_t fused_train_workspace_bytes(const tnn_mlp_desc *d, size_t M);
+// mlp.hip
+int backward128_from_loss(const tnn_mlp_desc *desc, const void *wprep_bwd, const void *interm_fwd, const float *targets, float loss_scale,
+                          float *loss_sum, void *dW, int dW_is_fp32, void *dLdx, size_t M, void *workspace, size_t workspace_bytes, hipStream_t s);
 
 } // namespace tnn
 
@@ -86,6 +89,9 @@ TNN_API int tnn_mlp_train_step_l2(const tnn_mlp_desc *desc, const void *d_prepar
     if (d_y && hipMemcpyAsync(d_y, y, mat, hipMemcpyDeviceToDevice, s) != hipSuccess) return fail(TNN_ERR_HIP, "copy of the network output failed");
     const size_t n = M * W;
     if (d_loss_sum) TNN_LAUNCH(zero_scalar_kernel, dim3(1), dim3(1), 0, s, d_loss_sum);
+    // width 128: the loss is part of the backward pass's first launch (dL/dy is never written)
+    if (W == 128) return backward128_from_loss(desc, d_prepared_bwd, interm_fwd, d_targets, loss_scale, d_loss_sum, d_dW, dW_is_fp32, d_dLdx, M, bwd_ws,
+                                               bwd_ws_bytes, s);
     size_t blocks = (n + 256 * 8 - 1) / (256 * 8);
     if (blocks > 2048) blocks = 2048;
     const float inv_n = 1.0f / (float)n;

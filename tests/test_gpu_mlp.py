@@ -399,7 +399,7 @@ def test_linearity_property_full_size(tnn, oracle):
 @pytest.mark.parametrize("W,n_hidden,act,out_act", [(64, 4, "relu", "none"), (64, 2, "relu", "none"), (64, 1, "sigmoid", "sigmoid"),
                                                     (32, 4, "relu", "relu"), (32, 5, "none", "none"), (16, 2, "relu", "none"),
                                                     (16, 1, "sigmoid", "none"), (64, 3, "none", "sigmoid"), (128, 2, "relu", "none"),
-                                                    (64, 6, "relu", "none")])
+                                                    (64, 6, "relu", "none"), (128, 3, "relu", "sigmoid"), (128, 1, "sigmoid", "relu")])
 def test_train_step_single_call(tnn, oracle, dtype, W, n_hidden, act, out_act):
     """tnn_mlp_train_step_l2 (one kernel for widths <= 64 and <= 4-5 hidden layers, separate kernels over
     workspace matrices otherwise) against forward + L2 + backward called one by one, and against the oracle."""

@@ -807,23 +807,41 @@ static int launch_backward128(const tnn_mlp_desc *d, const void *wprep_bwd, cons
     const size_t mat = M * W, per_mat = (size_t)4 * 8 * 64;
     auto k_top = targets ? mlp_layer_backward128_kernel<T, 2> : mlp_layer_backward128_kernel<T, 1>;
     auto k_mid = mlp_layer_backward128_kernel<T, 0>;
+    auto k_pair = mlp_layer_pair_backward128_kernel<T>;
     const float inv_n = 1.0f / (float)(M * W);
     for (auto k : {k_top, k_mid})
         if (hipFuncSetAttribute(reinterpret_cast<const void *>(k), hipFuncAttributeMaxDynamicSharedMemorySize, (int)LayerBwd128::lds_bytes) != hipSuccess)
             return fail(TNN_ERR_HIP, "cannot reserve %zu bytes of LDS", LayerBwd128::lds_bytes);
+    if (hipFuncSetAttribute(reinterpret_cast<const void *>(k_pair), hipFuncAttributeMaxDynamicSharedMemorySize, (int)LayerBwd128::lds_bytes) != hipSuccess)
+        return fail(TNN_ERR_HIP, "cannot reserve %zu bytes of LDS", LayerBwd128::lds_bytes);
     const T *fwd = static_cast<const T *>(interm_fwd);
     T *dl = static_cast<T *>(deltas);
-    for (int l = n_mats - 1; l >= 0; --l) {
+    const vec8 *wb = static_cast<const vec8 *>(wprep_bwd);
+    // the top layer by itself (it turns dL/dy or the loss into deltas first), then the layers below it two per launch, and
+    // the first matrix by itself when their number is odd
+    int l = n_mats - 1;
+    while (l >= 0) {
         const bool top = (l == n_mats - 1);
+        if (!top && l >= 1) {
+            T *delta_out = l > 1 ? dl + (size_t)(l - 2) * mat : static_cast<T *>(dLdx);
+            TNN_LAUNCH(k_pair, dim3((unsigned)p.n_chunks), dim3(kLayerBwdThreads), LayerBwd128::lds_bytes, s, wb + (size_t)l * per_mat,
+                       wb + (size_t)(l - 1) * per_mat, dl + (size_t)l * mat, fwd + (size_t)l * mat, fwd + (size_t)(l - 1) * mat,
+                       keep_top_delta ? dl + (size_t)(l - 1) * mat : (T *)nullptr, delta_out, partials, n_mats, l, d->activation,
+                       l > 1 ? d->activation : TNN_ACT_NONE, (long long)M, p.rows_per_chunk);
+            const int rc = check_launch("mlp_layer_pair_backward128_kernel");
+            if (rc) return rc;
+            l -= 2;
+            continue;
+        }
         const T *delta_in = top ? static_cast<const T *>(dLdy) : dl + (size_t)l * mat;
         T *delta_out = l > 0 ? dl + (size_t)(l - 1) * mat : static_cast<T *>(dLdx);
         const int gate = l > 0 ? d->activation : TNN_ACT_NONE;
-        TNN_LAUNCH((top ? k_top : k_mid), dim3((unsigned)p.n_chunks), dim3(kLayerBwdThreads), LayerBwd128::lds_bytes, s,
-                   (const vec8 *)wprep_bwd + (size_t)l * per_mat, delta_in, fwd + (size_t)l * mat, fwd + (size_t)n_mats * mat,
-                   (top && keep_top_delta) ? dl + (size_t)l * mat : (T *)nullptr, delta_out, partials, n_mats, l, gate, d->output_activation,
-                   (long long)M, p.rows_per_chunk, targets, loss_scale, inv_n, loss_sum);
+        TNN_LAUNCH((top ? k_top : k_mid), dim3((unsigned)p.n_chunks), dim3(kLayerBwdThreads), LayerBwd128::lds_bytes, s, wb + (size_t)l * per_mat,
+                   delta_in, fwd + (size_t)l * mat, fwd + (size_t)n_mats * mat, (top && keep_top_delta) ? dl + (size_t)l * mat : (T *)nullptr,
+                   delta_out, partials, n_mats, l, gate, d->output_activation, (long long)M, p.rows_per_chunk, targets, loss_scale, inv_n, loss_sum);
         const int rc = check_launch("mlp_layer_backward128_kernel");
         if (rc) return rc;
+        l -= 1;
     }
     const int n_elems = n_mats * W * W;
     TNN_LAUNCH((dw_reduce_kernel<T>), dim3(n_elems / 64), dim3(512), 0, s, partials, (int)(p.n_chunks * p.partials_per_chunk), n_elems,

@@ -102,42 +102,61 @@ __global__ void __launch_bounds__(kOrderThreads)
 }
 
 // Step 1b: turns the histograms into starting positions, in place. Bins are laid out in key order, and inside a bin the
-// workgroups in their own order. Workgroup g of this kernel owns bins [64 g, 64 g + 64).
-__global__ void __launch_bounds__(256)
+// workgroups in their own order. Workgroup g of this kernel owns bins [64 g, 64 g + 64). The prefix over the workgroups of
+// a bin is a chain of dependent LDS accesses, so the sixteen waves each take a sixteenth of the workgroups (lane = bin)
+// and the sixteen partial sums per bin are put together afterwards.
+constexpr int kScanThreads = 1024;
+constexpr int kScanParts = kScanThreads / 64;
+__global__ void __launch_bounds__(kScanThreads)
     order_scan_kernel(uint32_t *__restrict__ hist, const uint32_t *__restrict__ group_totals, int n_wg) {
-    extern __shared__ uint32_t tile[]; // [n_wg][64] counts, then 64 bin totals, then 4 wave sums
-    uint32_t *bin_total = tile + (size_t)n_wg * 64;
-    uint32_t *wave_sum = bin_total + 64;
-    const int g = blockIdx.x, tid = threadIdx.x;
+    extern __shared__ uint32_t tile[]; // [n_wg][64] counts, then [parts][64] partial sums, then 64 bin starts, then the wave sums
+    uint32_t *part_sum = tile + (size_t)n_wg * 64;
+    uint32_t *bin_start = part_sum + kScanParts * 64;
+    uint32_t *wave_sum = bin_start + 64;
+    const int g = blockIdx.x, tid = threadIdx.x, bin = tid & 63, part = tid >> 6;
     // everything in front of this run of bins
     uint32_t before = 0;
-    for (int e = tid; e < n_wg * kOrderGroups; e += 256) // coalesced, every load independent of the one before
+    for (int e = tid; e < n_wg * kOrderGroups; e += kScanThreads) // coalesced, every load independent of the one before
         before += ((e & (kOrderGroups - 1)) < g) ? group_totals[e] : 0u;
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) before += __shfl_down(before, off, 64);
-    if ((tid & 63) == 0) wave_sum[tid >> 6] = before;
-    for (int e = tid; e < n_wg * 64; e += 256) tile[e] = hist[(size_t)(e >> 6) * kOrderBins + 64 * g + (e & 63)];
+    if (bin == 0) wave_sum[part] = before;
+    for (int e = tid; e < n_wg * 64; e += kScanThreads) tile[e] = hist[(size_t)(e >> 6) * kOrderBins + 64 * g + (e & 63)];
     __syncthreads();
-    const uint32_t base = wave_sum[0] + wave_sum[1] + wave_sum[2] + wave_sum[3];
+    // exclusive prefix over this wave's workgroups of one bin (lanes on consecutive words: no bank conflicts)
+    const int per = (n_wg + kScanParts - 1) / kScanParts;
+    const int w_begin = part * per, w_end = (w_begin + per < n_wg) ? w_begin + per : n_wg;
+    uint32_t run = 0;
+    for (int w = w_begin; w < w_end; ++w) {
+        const uint32_t c = tile[w * 64 + bin];
+        tile[w * 64 + bin] = run;
+        run += c;
+    }
+    part_sum[part * 64 + bin] = run;
+    __syncthreads();
     if (tid < 64) {
-        // exclusive prefix over the workgroups of one bin (lanes on consecutive words: no bank conflicts)
-        uint32_t run = 0;
-        for (int w = 0; w < n_wg; ++w) {
-            const uint32_t c = tile[w * 64 + tid];
-            tile[w * 64 + tid] = run;
-            run += c;
+        uint32_t base = 0;
+#pragma unroll
+        for (int i = 0; i < kScanParts; ++i) base += wave_sum[i];
+        // the parts of a bin one after the other, then an exclusive prefix over the 64 bins
+        uint32_t total = 0;
+#pragma unroll
+        for (int i = 0; i < kScanParts; ++i) {
+            const uint32_t c = part_sum[i * 64 + tid];
+            part_sum[i * 64 + tid] = total;
+            total += c;
         }
-        // exclusive prefix over the 64 bins
-        uint32_t incl = run;
+        uint32_t incl = total;
 #pragma unroll
         for (int off = 1; off < 64; off <<= 1) {
             const uint32_t v = __shfl_up(incl, off, 64);
             if (tid >= off) incl += v;
         }
-        bin_total[tid] = base + incl - run;
+        bin_start[tid] = base + incl - total;
     }
     __syncthreads();
-    for (int e = tid; e < n_wg * 64; e += 256) hist[(size_t)(e >> 6) * kOrderBins + 64 * g + (e & 63)] = tile[e] + bin_total[e & 63];
+    for (int e = tid; e < n_wg * 64; e += kScanThreads)
+        hist[(size_t)(e >> 6) * kOrderBins + 64 * g + (e & 63)] = tile[e] + part_sum[((e >> 6) / per) * 64 + (e & 63)] + bin_start[e & 63];
 }
 
 // Step 1c: every point goes to the next free position of its bin (the workgroup's own counters, in LDS).
@@ -240,7 +259,7 @@ TNN_API int tnn_grid_order_points(const tnn_grid_desc *desc, const float *d_x, s
     uint32_t *hist = reinterpret_cast<uint32_t *>(static_cast<char *>(d_order) + p.record_bytes);
     uint32_t *groups = reinterpret_cast<uint32_t *>(static_cast<char *>(d_order) + p.record_bytes + p.hist_bytes);
     hipStream_t s = as_stream(stream);
-    const size_t scan_lds = ((size_t)p.n_wg * 64 + 64 + 4) * sizeof(uint32_t);
+    const size_t scan_lds = ((size_t)p.n_wg * 64 + kScanParts * 64 + 64 + kScanParts) * sizeof(uint32_t);
     if (scan_lds > 48 * 1024 &&
         hipFuncSetAttribute(reinterpret_cast<const void *>(order_scan_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)scan_lds) != hipSuccess)
         return fail(TNN_ERR_HIP, "cannot reserve %zu bytes of LDS", scan_lds);
@@ -248,7 +267,7 @@ TNN_API int tnn_grid_order_points(const tnn_grid_desc *desc, const float *d_x, s
     do {                                                                                                                               \
         TNN_LAUNCH((order_hist_kernel<D_>), dim3(p.n_wg), dim3(kOrderThreads), 0, s, d_x, (long long)M, p.chunk, hist, groups);         \
         if ((rc = check_launch("order_hist_kernel"))) return rc;                                                                       \
-        TNN_LAUNCH(order_scan_kernel, dim3(kOrderGroups), dim3(256), scan_lds, s, hist, (const uint32_t *)groups, p.n_wg);              \
+        TNN_LAUNCH(order_scan_kernel, dim3(kOrderGroups), dim3(kScanThreads), scan_lds, s, hist, (const uint32_t *)groups, p.n_wg);              \
         if ((rc = check_launch("order_scan_kernel"))) return rc;                                                                       \
         TNN_LAUNCH((order_scatter_kernel<D_>), dim3(p.n_wg), dim3(kOrderThreads), 0, s, d_x, (long long)M, p.chunk, (const uint32_t *)hist, records); \
         if ((rc = check_launch("order_scatter_kernel"))) return rc;                                                                    \

@@ -142,9 +142,19 @@ def test_captured_fused_grid_step_replays_like_eager(tnn):
             t.fill_(float("nan"))
         graph.replay()
         replayed = snapshot()
+        # Per-row results are bit-equal. Points of one cell take their places in the cell order by LDS atomics, so two runs put
+        # other rows into a tile and take the fp32 sums over the batch (loss, weight gradients, table gradients) in another
+        # order: those, and what Adam makes of them, agree to rounding.
         for name, a, b in zip(("y", "loss", "master", "forward weights", "backward weights", "gradient table"), eager, replayed):
-            if name == "gradient table":
+            if name == "y":
+                assert torch.equal(a, b), f"replay {it}: {name}"
+            elif name == "loss":
+                assert abs(float(a) - float(b)) <= 1e-5 * abs(float(a)), f"replay {it}: {name}"
+            elif name == "master":
+                assert torch.allclose(a, b, rtol=1e-5, atol=2e-6), f"replay {it}: {name}: {float((a - b).abs().max())}"
+            elif name == "gradient table":
                 assert torch.allclose(a, b, rtol=1e-4, atol=1e-6 * float(a.abs().max())), f"replay {it}: {name}"
             else:
-                assert torch.equal(a, b), f"replay {it}: {name}"
+                assert torch.allclose(a.float(), b.float(), rtol=2 ** -7, atol=1e-5), f"replay {it}: {name}"
+                assert float((a.view(torch.int16) != b.view(torch.int16)).float().mean()) < 0.01, f"replay {it}: {name}: too many weights rounded the other way"
         assert float(eager[1]) > 0

@@ -16,7 +16,7 @@ calls so that the clocks are up before the declared warm-up, (3) --warmup untime
 of EXACTLY --steps steps, enqueued back to back on one stream with a HIP event between repetitions and one synchronisation
 at each end; `ms_per_step` is the median repetition and `ms_per_step_reps` lists all of them.
 
---workload train|infer|grid|train_fb|grid_mlp|grid_train runs one workload on its own (the form the profiles under profiles/
+--workload train|infer|grid|train_fb|train_w128|grid_mlp|grid_train runs one workload on its own (the form the profiles under profiles/
 were collected with); its line has the same top-level fields.
 """
 import argparse
@@ -60,7 +60,7 @@ def parse():
     ap.add_argument("--reps", type=int, default=5, help="repetitions of --steps timed steps; the median is reported")
     ap.add_argument("--prewarm-ms", type=float, default=300.0,
                     help="untimed calls for this long before the declared warm-up (a fresh process starts at idle clocks)")
-    ap.add_argument("--workload", default="all", choices=["all", "train", "train_fb", "infer", "grid", "grid_mlp", "grid_train"])
+    ap.add_argument("--workload", default="all", choices=["all", "train", "train_fb", "train_w128", "infer", "grid", "grid_mlp", "grid_train"])
     ap.add_argument("--batch-log2", type=int, default=None)
     ap.add_argument("--packed-scatter", action="store_true",
                     help="grid_train only: gradient table in fp16 with one packed atomic per feature pair (tnn_grid_backward_packed)")
@@ -89,25 +89,26 @@ def _timed_loop(fn, budget_s):
     return n, time.perf_counter() - t0
 
 
-def cpu_baseline_train(oracle, W, n_mats, budget_s=12.0):
+def cpu_baseline_train(oracle, W, n_mats, budget_s=12.0, fp16=False):
     import numpy as np
-    from tolerances import BF16
+    from tolerances import BF16, FP16
 
+    T = FP16 if fp16 else BF16
     rng = np.random.default_rng(0)
     lim = np.sqrt(6.0 / (2 * W))
-    w = oracle.round(rng.uniform(-lim, lim, (n_mats, W, W)), BF16)
+    w = oracle.round(rng.uniform(-lim, lim, (n_mats, W, W)), T)
     M = 1 << 14
-    x = oracle.round(rng.uniform(-1, 1, (M, W)), BF16)
+    x = oracle.round(rng.uniform(-1, 1, (M, W)), T)
     tg = rng.uniform(0, 1, (M, W)).astype(np.float32)
 
     def step():
-        interm = oracle.mlp_forward_T(BF16, W, n_mats, "relu", "none", w, x)
-        _, g = oracle.l2_loss(BF16, interm[-1], tg, 1.0)
-        oracle.mlp_backward_T(BF16, W, n_mats, "relu", "none", w, interm, g, want_dx=False, round_dw=False)
+        interm = oracle.mlp_forward_T(T, W, n_mats, "relu", "none", w, x)
+        _, g = oracle.l2_loss(T, interm[-1], tg, 128.0 if fp16 else 1.0)
+        oracle.mlp_backward_T(T, W, n_mats, "relu", "none", w, interm, g, want_dx=False, round_dw=False)
 
     n, dt = _timed_loop(step, budget_s)
     return {"value": M * n / dt, "unit": "samples/s", "cores": oracle.num_threads(), "kind": "port",
-            "sample": f"{n} training steps (forward, L2, backward with dW) of {M} rows each, w64 / 4 hidden layers, bf16 rounding points, OpenMP over rows"}
+            "sample": f"{n} training steps (forward, L2, backward with dW) of {M} rows each, w{W} / {n_mats - 1} hidden layers, {'fp16' if fp16 else 'bf16'} rounding points, OpenMP over rows"}
 
 
 def cpu_baseline_infer(oracle, W, n_mats, budget_s=12.0):
@@ -530,6 +531,55 @@ class Bench:
         return out, w
 
     # --------------------------------------------------------------------------------------------------------------
+    def leg_train_w128(self):
+        # BASELINE config 3's widest network: width 128, 8 hidden layers, fp16, 2^20 rows. Its nine matrices do not fit one
+        # kernel: a forward pass that stores the activations, the top layer's backward launch with the loss in it, then
+        # one backward launch per two layers. Parity at this size: tests/test_gpu_mlp.py::test_baseline_config_3_full_size.
+        np, torch, t, lib = self.np, self.torch, self.t, self.lib
+        from tiny_dpcpp_nn.cabi import ptr
+        from tolerances import FP16, FP32
+        W, n_hidden = 128, 8
+        n_mats = n_hidden + 1
+        M = 1 << (self.args.batch_log2 or 20)
+        desc = t.mlp_desc(FP16, W, n_hidden, "relu", "none")
+        rng = np.random.default_rng(42)
+        lim = np.sqrt(6.0 / (2 * W))
+        w = rng.uniform(-lim, lim, (n_mats, W, W)).astype(np.float32)
+        gen = torch.Generator(device=t.dev).manual_seed(1234)
+        x = (torch.rand((M, W), device=t.dev, generator=gen) * 2 - 1).to(torch.float16)
+        targets = torch.rand((M, W), device=t.dev, generator=gen)
+        master = t.pack(FP32, W, n_mats, torch.from_numpy(w.reshape(-1)).to(t.dev))
+        pf, pb = t.prepare_packed(desc, master, src_is_fp32=True)
+        m, v = torch.zeros_like(master), torch.zeros_like(master)
+        loss = torch.zeros(1, device=t.dev)
+        ws_bytes = lib.tnn_mlp_train_step_workspace_bytes(ctypes.byref(desc), M)
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=t.dev)
+        s, d = t.stream(), ctypes.byref(desc)
+        a = (ptr(pf), ptr(pb), ptr(x), ptr(targets), ptr(loss), ptr(master), ptr(m), ptr(v), ptr(ws))
+
+        def step(i):
+            if lib.tnn_mlp_train_step_l2_adam(d, a[0], a[1], a[2], a[3], 128.0, None, a[4], a[5], a[6], a[7], i + 1, 1e-3, 0.9, 0.99, 1e-15, None,
+                                              None, M, a[8], ws_bytes, None, s):
+                raise RuntimeError(lib.tnn_last_error())
+
+        step(0)
+        torch.cuda.synchronize()
+        loss0 = float(loss.item())
+        timer = self.timer()
+        timer.n = 1
+        tm = timer.run(step)
+        flops = 3 * 2 * M * W * W * n_mats
+        lg = int(np.log2(M))
+        ach = flops / (tm["ms"] * 1e-3) / 1e12
+        roof = {"bound": "mfma", "achieved": ach, "peak": PEAK_MFMA_BF16, "unit": "TFLOP/s", "frac": ach / PEAK_MFMA_BF16, "traffic": None,
+                "kernel": "whole step: mlp_forward_stream_kernel, mlp_layer_backward128_kernel (top layer + loss), "
+                          "mlp_layer_pair_backward128_kernel x (n_hidden / 2), dw_reduce_kernel, mlp_adam_update_kernel",
+                "kernel_ms": tm["ms"], "algorithmic_flops_per_launch": flops}
+        return line("fused-MLP training samples/s (w128, 8 hidden layers, fp16, batch 2^20); % fp16 MFMA peak", "samples/s", "f16",
+                    f"training step: w128, 8 hidden layers (9 matmuls), ReLU/linear, fp16, batch 2^{lg}, L2 loss, Adam on fp32 masters (BASELINE config 3, widest)",
+                    M, tm, self.K, self.Wm, self.args, roof, {"loss_first": loss0, "loss_last": float(loss.item())}), W, n_mats
+
+    # --------------------------------------------------------------------------------------------------------------
     def leg_train_fb(self, c):
         # The reference's own training step (Trainer::training_step, include/trainer.h:23-46): a forward pass that stores every
         # activation, then a backward pass that returns the weight gradients, the deltas and dL/dx. No loss, no optimizer.
@@ -742,6 +792,11 @@ def main():
             out["infer"] = sub(inf)
         else:
             out = inf
+    if wl == "train_w128":
+        out, W128, n_mats128 = b.leg_train_w128()
+        out.update({"parity_checked": False, "parity": None})
+        if do_cpu:
+            out["cpu_baseline"] = cpu_baseline_train(oracle, W128, n_mats128, fp16=True)
     if wl == "train_fb":
         out = b.leg_train_fb(c)
         if do_cpu:

@@ -183,11 +183,11 @@ __global__ void __launch_bounds__(kStreamThreads, 1)
         long long row[R];
         bool valid[R];
         vec8 cur[R][NK];
-        unsigned int st_off[R][NK];
+        unsigned int st_base[R];
         auto put = [&](int t, T *dst) __attribute__((always_inline)) {
             if constexpr (STAGED != 0) {
                 TL::stage(cur[t], my_stage, j, h);
-                TL::template store_staged<(STAGED == 2 ? kStreamingStore : 0)>(my_stage, lane, TL::rows_of(dst, M), st_off[t]);
+                TL::template store_staged_at<(STAGED == 2 ? kStreamingStore : 0)>(my_stage, lane, TL::rows_of(dst, M), st_base[t]);
             } else {
                 TL::store(cur[t], dst, row[t], h, valid[t]);
             }
@@ -196,7 +196,7 @@ __global__ void __launch_bounds__(kStreamThreads, 1)
         for (int t = 0; t < R; ++t) {
             row[t] = r * ROUND + (wave * R + t) * 32 + j;
             valid[t] = row[t] < M;
-            if constexpr (STAGED != 0) TL::row_offsets(st_off[t], r * (ROUND / 32) + wave * R + t, lane, M);
+            if constexpr (STAGED != 0) st_base[t] = TL::staged_base(r * (ROUND / 32) + wave * R + t, lane);
             TL::load(cur[t], x, row[t], h, valid[t]);
             if (STORE_INTERM) put(t, out);
         }

@@ -195,6 +195,20 @@ template <typename T, int W> struct Tile {
                                                    rows, o[i], 0, AUX);
     }
 
+    // The same store from one offset per tile (that of the lane's 16 bytes in the first of its rows) and a constant per
+    // instruction. Rows past the end of the matrix need no flag: their offsets lie past the end of the buffer resource and the
+    // range check drops them (the resource covers less than 2^31 bytes, so an offset cannot wrap back into range).
+    static __device__ __forceinline__ unsigned int staged_base(long long tile, int lane) {
+        return (unsigned int)((tile * 32 + lane / LPR) * (W * (long long)sizeof(T))) + (lane % LPR) * 16;
+    }
+    template <int AUX = 0>
+    static __device__ __forceinline__ void store_staged_at(const unsigned char *tile_lds, int lane, __amdgpu_buffer_rsrc_t rows, unsigned int base) {
+#pragma unroll
+        for (int i = 0; i < NK; ++i)
+            __builtin_amdgcn_raw_buffer_store_b128(*reinterpret_cast<const u32x4 *>(tile_lds + (i * RPI + lane / LPR) * PITCH + (lane % LPR) * 16),
+                                                   rows, base, i * RPI * W * (int)sizeof(T), AUX);
+    }
+
     static constexpr int NF = NI * NK; // weight fragments per matrix and lane
 
     // The lane's NF operand fragments of matrix l (LDS or global, already in operand order).

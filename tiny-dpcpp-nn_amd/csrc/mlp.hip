@@ -158,7 +158,7 @@ constexpr int kStreamTiles = 2;
 template <typename T, int W, int ACT, bool STORE_INTERM, int STAGED = 0>
 __global__ void __launch_bounds__(kStreamThreads, 1)
     mlp_forward_stream_kernel(const typename Storage<T>::vec8 *__restrict__ wprep, const T *__restrict__ x, T *__restrict__ out,
-                              int n_mats, int out_act, long long M) {
+                              int n_mats, int out_act, long long M, int store_input) {
     typedef Tile<T, W> TL;
     typedef typename Storage<T>::vec8 vec8;
     constexpr int NK = TL::NK, NI = TL::NI, R = kStreamTiles;
@@ -198,7 +198,7 @@ __global__ void __launch_bounds__(kStreamThreads, 1)
             valid[t] = row[t] < M;
             if constexpr (STAGED != 0) st_base[t] = TL::staged_base(r * (ROUND / 32) + wave * R + t, lane);
             TL::load(cur[t], x, row[t], h, valid[t]);
-            if (STORE_INTERM) put(t, out);
+            if (STORE_INTERM && store_input) put(t, out); // (a training step reads the input where it is: it leaves matrix 0 unwritten)
         }
         const bool more_rounds = r + gridDim.x < n_rounds;
         for (int l = 0; l < n_mats; ++l) {
@@ -612,7 +612,8 @@ static long long stream_grid(const void *kernel, size_t lds_bytes, size_t M, int
 }
 
 template <typename T, int W, int ACT, bool STORE_INTERM, int THREADS>
-static int launch_forward_v(const tnn_mlp_desc *d, const void *wprep, const void *x, void *out, size_t M, hipStream_t s, int per_cu) {
+static int launch_forward_v(const tnn_mlp_desc *d, const void *wprep, const void *x, void *out, size_t M, hipStream_t s, int per_cu,
+                            bool store_input = true) { // store_input = false: the width-128 streaming route may leave matrix 0 of `out` unwritten
     typedef typename Storage<T>::vec8 vec8;
     const int n_mats = d->n_hidden_layers + 1;
     const size_t wbytes = prepared_elems(d) * sizeof(T);
@@ -640,7 +641,7 @@ static int launch_forward_v(const tnn_mlp_desc *d, const void *wprep, const void
             if (hipFuncSetAttribute(reinterpret_cast<const void *>(k), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_k) != hipSuccess)
                 return fail(TNN_ERR_HIP, "cannot reserve %zu bytes of LDS", lds_k);
             TNN_LAUNCH(k, dim3((unsigned)g), dim3(kStreamThreads), lds_k, s, (const vec8 *)wprep, (const T *)x, (T *)out, n_mats,
-                       d->output_activation, (long long)M);
+                       d->output_activation, (long long)M, store_input ? 1 : 0);
             return check_launch("mlp_forward_stream_kernel");
         }
     }
@@ -693,7 +694,7 @@ static int launch_forward_v(const tnn_mlp_desc *d, const void *wprep, const void
 // measured faster than 256-thread workgroups at higher counts and than variants that hold the next matrix's
 // fragments in registers.
 template <typename T, int W, int ACT, bool STORE_INTERM>
-static int launch_forward_act(const tnn_mlp_desc *d, const void *wprep, const void *x, void *out, size_t M, hipStream_t s) {
+static int launch_forward_act(const tnn_mlp_desc *d, const void *wprep, const void *x, void *out, size_t M, hipStream_t s, bool store_input = true) {
     if constexpr (W <= 64) {
         // From two tiles per wave on a full chip: one workgroup of 16 waves per CU instead of two of 8, so that the weights
         // are staged once per CU (inference at 2^18 rows, w64 with 4 hidden layers: 13.7 -> 13.2 us); below that the
@@ -703,15 +704,15 @@ static int launch_forward_act(const tnn_mlp_desc *d, const void *wprep, const vo
         if (di.ok && (M + 31) / 32 >= (size_t)di.n_cu * 32 && staged_bytes <= 160 * 1024)
             return launch_forward_v<T, W, ACT, STORE_INTERM, 1024>(d, wprep, x, out, M, s, 1);
     }
-    return launch_forward_v<T, W, ACT, STORE_INTERM, 512>(d, wprep, x, out, M, s, 2);
+    return launch_forward_v<T, W, ACT, STORE_INTERM, 512>(d, wprep, x, out, M, s, 2, store_input);
 }
 
 template <typename T, int W, bool STORE_INTERM>
-static int launch_forward(const tnn_mlp_desc *d, const void *wprep, const void *x, void *out, size_t M, hipStream_t s) {
+static int launch_forward(const tnn_mlp_desc *d, const void *wprep, const void *x, void *out, size_t M, hipStream_t s, bool store_input = true) {
     switch (d->activation) {
-    case TNN_ACT_RELU: return launch_forward_act<T, W, TNN_ACT_RELU, STORE_INTERM>(d, wprep, x, out, M, s);
-    case TNN_ACT_SIGMOID: return launch_forward_act<T, W, TNN_ACT_SIGMOID, STORE_INTERM>(d, wprep, x, out, M, s);
-    default: return launch_forward_act<T, W, TNN_ACT_NONE, STORE_INTERM>(d, wprep, x, out, M, s);
+    case TNN_ACT_RELU: return launch_forward_act<T, W, TNN_ACT_RELU, STORE_INTERM>(d, wprep, x, out, M, s, store_input);
+    case TNN_ACT_SIGMOID: return launch_forward_act<T, W, TNN_ACT_SIGMOID, STORE_INTERM>(d, wprep, x, out, M, s, store_input);
+    default: return launch_forward_act<T, W, TNN_ACT_NONE, STORE_INTERM>(d, wprep, x, out, M, s, store_input);
     }
 }
 
@@ -799,7 +800,7 @@ static int launch_dw(const tnn_mlp_desc *d, const void *interm_bwd, const void *
 template <typename T>
 static int launch_backward128(const tnn_mlp_desc *d, const void *wprep_bwd, const void *dLdy, const void *interm_fwd, void *deltas,
                               bool keep_top_delta, void *dW, int dW_is_fp32, void *dLdx, size_t M, float *partials, hipStream_t s,
-                              const float *targets = nullptr, float loss_scale = 0.0f, float *loss_sum = nullptr) {
+                              const float *targets = nullptr, float loss_scale = 0.0f, float *loss_sum = nullptr, const void *x0 = nullptr) {
     typedef typename Storage<T>::vec8 vec8;
     constexpr int W = 128;
     const int n_mats = d->n_hidden_layers + 1;
@@ -815,6 +816,7 @@ static int launch_backward128(const tnn_mlp_desc *d, const void *wprep_bwd, cons
     if (hipFuncSetAttribute(reinterpret_cast<const void *>(k_pair), hipFuncAttributeMaxDynamicSharedMemorySize, (int)LayerBwd128::lds_bytes) != hipSuccess)
         return fail(TNN_ERR_HIP, "cannot reserve %zu bytes of LDS", LayerBwd128::lds_bytes);
     const T *fwd = static_cast<const T *>(interm_fwd);
+    const T *input0 = x0 ? static_cast<const T *>(x0) : fwd; // the first matrix's input: the caller's x, or its copy in front of the activations
     T *dl = static_cast<T *>(deltas);
     const vec8 *wb = static_cast<const vec8 *>(wprep_bwd);
     // the top layer by itself (it turns dL/dy or the loss into deltas first), then the layers below it two per launch, and
@@ -825,7 +827,7 @@ static int launch_backward128(const tnn_mlp_desc *d, const void *wprep_bwd, cons
         if (!top && l >= 1) {
             T *delta_out = l > 1 ? dl + (size_t)(l - 2) * mat : static_cast<T *>(dLdx);
             TNN_LAUNCH(k_pair, dim3((unsigned)p.n_chunks), dim3(kLayerBwdThreads), LayerBwd128::lds_bytes, s, wb + (size_t)l * per_mat,
-                       wb + (size_t)(l - 1) * per_mat, dl + (size_t)l * mat, fwd + (size_t)l * mat, fwd + (size_t)(l - 1) * mat,
+                       wb + (size_t)(l - 1) * per_mat, dl + (size_t)l * mat, fwd + (size_t)l * mat, l > 1 ? fwd + (size_t)(l - 1) * mat : input0,
                        keep_top_delta ? dl + (size_t)(l - 1) * mat : (T *)nullptr, delta_out, partials, n_mats, l, d->activation,
                        l > 1 ? d->activation : TNN_ACT_NONE, (long long)M, p.rows_per_chunk);
             const int rc = check_launch("mlp_layer_pair_backward128_kernel");
@@ -837,7 +839,7 @@ static int launch_backward128(const tnn_mlp_desc *d, const void *wprep_bwd, cons
         T *delta_out = l > 0 ? dl + (size_t)(l - 1) * mat : static_cast<T *>(dLdx);
         const int gate = l > 0 ? d->activation : TNN_ACT_NONE;
         TNN_LAUNCH((top ? k_top : k_mid), dim3((unsigned)p.n_chunks), dim3(kLayerBwdThreads), LayerBwd128::lds_bytes, s, wb + (size_t)l * per_mat,
-                   delta_in, fwd + (size_t)l * mat, fwd + (size_t)n_mats * mat, (top && keep_top_delta) ? dl + (size_t)l * mat : (T *)nullptr,
+                   delta_in, l > 0 ? fwd + (size_t)l * mat : input0, fwd + (size_t)n_mats * mat, (top && keep_top_delta) ? dl + (size_t)l * mat : (T *)nullptr,
                    delta_out, partials, n_mats, l, gate, d->output_activation, (long long)M, p.rows_per_chunk, targets, loss_scale, inv_n, loss_sum);
         const int rc = check_launch("mlp_layer_backward128_kernel");
         if (rc) return rc;
@@ -849,9 +851,16 @@ static int launch_backward128(const tnn_mlp_desc *d, const void *wprep_bwd, cons
     return check_launch("dw_reduce_kernel");
 }
 
-// For tnn_mlp_train_step_l2 on width 128: loss and backward pass over stored activations, the loss folded into the top
-// layer's launch. Workspace as tnn_mlp_backward's.
-int backward128_from_loss(const tnn_mlp_desc *desc, const void *wprep_bwd, const void *interm_fwd, const float *targets, float loss_scale,
+// For tnn_mlp_train_step_l2 on width 128. The forward pass with stored activations that does not copy the input in front of
+// them where its kernel can leave that out (2^20 rows: 268 MB less to write), ...
+int forward128_for_training(const tnn_mlp_desc *desc, const void *wprep, const void *x, void *interm_fwd, size_t M, hipStream_t s) {
+    if (desc->dtype == TNN_BF16) return launch_forward<bf16_t, 128, true>(desc, wprep, x, interm_fwd, M, s, false);
+    return launch_forward<fp16_t, 128, true>(desc, wprep, x, interm_fwd, M, s, false);
+}
+
+// ... and loss and backward pass over those activations, the loss folded into the top layer's launch and the first matrix's
+// input read from `x`. Workspace as tnn_mlp_backward's.
+int backward128_from_loss(const tnn_mlp_desc *desc, const void *wprep_bwd, const void *x, const void *interm_fwd, const float *targets, float loss_scale,
                           float *loss_sum, void *dW, int dW_is_fp32, void *dLdx, size_t M, void *workspace, size_t workspace_bytes, hipStream_t s) {
     const DwPlan p = dw_plan(desc, M);
     const size_t partial_rounded = (p.partial_bytes + 255) & ~(size_t)255;
@@ -862,9 +871,9 @@ int backward128_from_loss(const tnn_mlp_desc *desc, const void *wprep_bwd, const
     void *deltas = reinterpret_cast<void *>(base + partial_rounded);
     if (desc->dtype == TNN_BF16)
         return launch_backward128<bf16_t>(desc, wprep_bwd, nullptr, interm_fwd, deltas, false, dW, dW_is_fp32, dLdx, M, partials, s, targets, loss_scale,
-                                          loss_sum);
+                                          loss_sum, x);
     return launch_backward128<fp16_t>(desc, wprep_bwd, nullptr, interm_fwd, deltas, false, dW, dW_is_fp32, dLdx, M, partials, s, targets, loss_scale,
-                                      loss_sum);
+                                      loss_sum, x);
 }
 
 #define TNN_DISPATCH_TW(desc, CALL)                                                          \

@@ -39,7 +39,8 @@ int fused_train_step(const tnn_mlp_desc *d, const void *wf, const void *wb, cons
                      hipStream_t s);
 size_t fused_train_workspace_bytes(const tnn_mlp_desc *d, size_t M);
 // mlp.hip
-int backward128_from_loss(const tnn_mlp_desc *desc, const void *wprep_bwd, const void *interm_fwd, const float *targets, float loss_scale,
+int forward128_for_training(const tnn_mlp_desc *desc, const void *wprep, const void *x, void *interm_fwd, size_t M, hipStream_t s);
+int backward128_from_loss(const tnn_mlp_desc *desc, const void *wprep_bwd, const void *x, const void *interm_fwd, const float *targets, float loss_scale,
                           float *loss_sum, void *dW, int dW_is_fp32, void *dLdx, size_t M, void *workspace, size_t workspace_bytes, hipStream_t s);
 
 } // namespace tnn
@@ -84,13 +85,13 @@ TNN_API int tnn_mlp_train_step_l2(const tnn_mlp_desc *desc, const void *d_prepar
     void *bwd_ws = reinterpret_cast<void *>(base);
     const size_t bwd_ws_bytes = align256(tnn_mlp_backward_workspace_bytes(desc, M));
 
-    if ((rc = tnn_mlp_forward(desc, d_prepared_fwd, d_x, interm_fwd, M, stream))) return rc;
+    if ((rc = (W == 128 ? forward128_for_training(desc, d_prepared_fwd, d_x, interm_fwd, M, s) : tnn_mlp_forward(desc, d_prepared_fwd, d_x, interm_fwd, M, stream)))) return rc;
     const void *y = static_cast<const char *>(interm_fwd) + (size_t)n_mats * mat;
     if (d_y && hipMemcpyAsync(d_y, y, mat, hipMemcpyDeviceToDevice, s) != hipSuccess) return fail(TNN_ERR_HIP, "copy of the network output failed");
     const size_t n = M * W;
     if (d_loss_sum) TNN_LAUNCH(zero_scalar_kernel, dim3(1), dim3(1), 0, s, d_loss_sum);
     // width 128: the loss is part of the backward pass's first launch (dL/dy is never written)
-    if (W == 128) return backward128_from_loss(desc, d_prepared_bwd, interm_fwd, d_targets, loss_scale, d_loss_sum, d_dW, dW_is_fp32, d_dLdx, M, bwd_ws,
+    if (W == 128) return backward128_from_loss(desc, d_prepared_bwd, d_x, interm_fwd, d_targets, loss_scale, d_loss_sum, d_dW, dW_is_fp32, d_dLdx, M, bwd_ws,
                                                bwd_ws_bytes, s);
     size_t blocks = (n + 256 * 8 - 1) / (256 * 8);
     if (blocks > 2048) blocks = 2048;

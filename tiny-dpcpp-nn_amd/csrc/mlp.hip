@@ -307,114 +307,6 @@ __global__ void __launch_bounds__(kFwdThreads)
     }
 }
 
-// Delta propagation with the matrices streamed through LDS (same scheme as mlp_forward_stream_kernel; the matrices are
-// visited from the last one down). The forward activation that gates a layer's deltas is loaded after the layer's
-// MFMAs, into the registers the consumed deltas leave free.
-template <typename T, int W>
-__global__ void __launch_bounds__(kStreamThreads, 1)
-    mlp_backward_stream_kernel(const typename Storage<T>::vec8 *__restrict__ wprep_bwd, const T *__restrict__ dLdy,
-                               const T *__restrict__ interm_fwd, T *__restrict__ interm_bwd, T *__restrict__ dLdx, int n_mats,
-                               int act, int out_act, long long M) {
-    typedef Tile<T, W> TL;
-    typedef typename Storage<T>::vec8 vec8;
-    constexpr int NK = TL::NK, NI = TL::NI, R = kStreamTiles;
-    constexpr int per_mat = NI * NK * kWaveSize;
-    constexpr int SHARE = per_mat / kStreamThreads;
-    extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
-    vec8 *lds = reinterpret_cast<vec8 *>(smem_raw);
-
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int j = lane & 31, h = lane >> 5;
-    constexpr int ROUND = (kStreamThreads / 64) * R * 32;
-    const long long n_rounds = (M + ROUND - 1) / ROUND;
-    const size_t mat = (size_t)M * W;
-    const int steps = n_mats - 1 + (dLdx ? 1 : 0); // step s multiplies by the transpose of matrix n_mats - 1 - s
-
-    vec8 st[SHARE];
-    {
-        const vec8 *first = wprep_bwd + (size_t)(n_mats - 1) * per_mat;
-#pragma unroll
-        for (int i = 0; i < SHARE; ++i) lds[threadIdx.x + kStreamThreads * i] = first[threadIdx.x + kStreamThreads * i];
-    }
-    int b = 0;
-
-    for (long long r = blockIdx.x; r < n_rounds; r += gridDim.x) {
-        long long row[R];
-        bool valid[R];
-        vec8 cur[R][NK];
-#pragma unroll
-        for (int t = 0; t < R; ++t) {
-            row[t] = r * ROUND + (wave * R + t) * 32 + j;
-            valid[t] = row[t] < M;
-            TL::load(cur[t], dLdy, row[t], h, valid[t]);
-            if (out_act != TNN_ACT_NONE) { // derivative of the output activation, on the T tile (kernel_esimd.h:193-201)
-                vec8 fwd[NK];
-                TL::load(fwd, interm_fwd + (size_t)n_mats * mat, row[t], h, valid[t]);
-#pragma unroll
-                for (int kb = 0; kb < NK; ++kb) {
-                    f32x8 v;
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) {
-                        const float g = (float)cur[t][kb][e], f = (float)fwd[kb][e];
-                        v[e] = (out_act == TNN_ACT_RELU) ? ((f <= 0.0f) ? 0.0f : g) : as_fp32(g * (f * (1.0f - f)));
-                    }
-                    cur[t][kb] = __builtin_convertvector(v, vec8);
-                }
-            }
-            if (interm_bwd) TL::store(cur[t], interm_bwd + (size_t)(n_mats - 1) * mat, row[t], h, valid[t]);
-        }
-        const bool more_rounds = r + gridDim.x < n_rounds;
-        for (int sidx = 0; sidx < steps; ++sidx) {
-            const int l = n_mats - 1 - sidx; // matrix of this step; its result is delta_{l-1} (or dL/dx for l == 0)
-            __syncthreads();
-            const bool last = sidx + 1 == steps;
-            const bool stage = !last || more_rounds;
-            const vec8 *next = wprep_bwd + (size_t)(last ? n_mats - 1 : l - 1) * per_mat;
-            if (stage) {
-#pragma unroll
-                for (int i = 0; i < SHARE; ++i) st[i] = next[threadIdx.x + kStreamThreads * i];
-            }
-            f32x16 acc[R][NI];
-#pragma unroll
-            for (int t = 0; t < R; ++t)
-#pragma unroll
-                for (int a = 0; a < NI; ++a) acc[t][a] = f32x16{};
-            const vec8 *w = lds + b * per_mat + lane;
-#pragma unroll
-            for (int kb = 0; kb < NK; ++kb) {
-#pragma unroll
-                for (int a = 0; a < NI; ++a) {
-                    const vec8 frag = w[(a * NK + kb) * kWaveSize];
-#pragma unroll
-                    for (int t = 0; t < R; ++t) acc[t][a] = Storage<T>::mfma(frag, cur[t][kb], acc[t][a]);
-                }
-            }
-            const bool gated = l > 0 && act != TNN_ACT_NONE;
-            if (stage) {
-#pragma unroll
-                for (int i = 0; i < SHARE; ++i) lds[(b ^ 1) * per_mat + threadIdx.x + kStreamThreads * i] = st[i];
-            }
-#pragma unroll
-            for (int t = 0; t < R; ++t) {
-                vec8 fwd[NK]; // takes the registers of the tile's consumed deltas
-                if (gated) TL::load(fwd, interm_fwd + (size_t)l * mat, row[t], h, valid[t]);
-                if (gated && act == TNN_ACT_RELU)
-                    TL::template bwd_repack<TNN_ACT_RELU>(cur[t], acc[t], fwd);
-                else if (gated)
-                    TL::template bwd_repack<TNN_ACT_SIGMOID>(cur[t], acc[t], fwd);
-                else
-                    TL::template repack<TNN_ACT_NONE>(cur[t], acc[t]);
-                if (l > 0) {
-                    if (interm_bwd) TL::store(cur[t], interm_bwd + (size_t)(l - 1) * mat, row[t], h, valid[t]);
-                } else {
-                    TL::store(cur[t], dLdx, row[t], h, valid[t]);
-                }
-            }
-            b ^= 1;
-        }
-    }
-}
-
 // ------------------------------------------------------------------------------------------
 // Weight gradients: dW_l[n][k] = sum_m delta_l[m][n] * a_l[m][k]   (kernel_esimd.h:230-239)
 // ------------------------------------------------------------------------------------------
@@ -716,6 +608,8 @@ static int launch_forward(const tnn_mlp_desc *d, const void *wprep, const void *
     }
 }
 
+// Delta propagation and (launch_dw) weight gradients as separate passes: widths up to 64 with more matrices than the
+// kernel that forms both keeps on chip. Width 128 has launch_backward128.
 template <typename T, int W>
 static int launch_backward(const tnn_mlp_desc *d, const void *wprep_bwd, const void *dLdy, const void *interm_fwd,
                            void *interm_bwd, void *dLdx, size_t M, hipStream_t s) {
@@ -735,17 +629,6 @@ static int launch_backward(const tnn_mlp_desc *d, const void *wprep_bwd, const v
         TNN_LAUNCH(k, dim3((unsigned)blocks), dim3(kFwdThreads), wbytes, s, (const vec8 *)wprep_bwd,
                            (const T *)dLdy, (const T *)interm_fwd, (T *)interm_bwd, (T *)dLdx, n_mats, d->activation,
                            d->output_activation, (long long)M);
-    } else if constexpr (W == 128) { // stream the matrices through LDS, one layer at a time
-        constexpr size_t lds = 2 * (size_t)Tile<T, W>::NI * Tile<T, W>::NK * kWaveSize * sizeof(vec8);
-        constexpr long long round = (kStreamThreads / 64) * kStreamTiles * 32;
-        long long g = ((long long)M + round - 1) / round;
-        if (g > di.n_cu) g = di.n_cu;
-        auto k = mlp_backward_stream_kernel<T, W>;
-        if (hipFuncSetAttribute(reinterpret_cast<const void *>(k), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
-            return fail(TNN_ERR_HIP, "cannot reserve %zu bytes of LDS", lds);
-        TNN_LAUNCH(k, dim3((unsigned)g), dim3(kStreamThreads), lds, s, (const vec8 *)wprep_bwd, (const T *)dLdy, (const T *)interm_fwd,
-                   (T *)interm_bwd, (T *)dLdx, n_mats, d->activation, d->output_activation, (long long)M);
-        return check_launch("mlp_backward_stream_kernel");
     } else {
         const long long blocks = stream_grid(reinterpret_cast<const void *>(mlp_backward_kernel<T, W, false>), 0, M, di.n_cu);
         TNN_LAUNCH((mlp_backward_kernel<T, W, false>), dim3((unsigned)blocks), dim3(kFwdThreads), 0, s,
@@ -895,6 +778,24 @@ int backward128_from_loss(const tnn_mlp_desc *desc, const void *wprep_bwd, const
         }                                                                                    \
     } while (0)
 
+// the widths below 128 (check_mlp_desc has let nothing else through)
+#define TNN_DISPATCH_TW_UP_TO_64(desc, CALL)                                                 \
+    do {                                                                                     \
+        if ((desc)->dtype == TNN_BF16) {                                                     \
+            switch ((desc)->width) {                                                         \
+            case 16: { typedef bf16_t T_; constexpr int W_ = 16; CALL; } break;              \
+            case 32: { typedef bf16_t T_; constexpr int W_ = 32; CALL; } break;              \
+            default: { typedef bf16_t T_; constexpr int W_ = 64; CALL; } break;              \
+            }                                                                                \
+        } else {                                                                             \
+            switch ((desc)->width) {                                                         \
+            case 16: { typedef fp16_t T_; constexpr int W_ = 16; CALL; } break;              \
+            case 32: { typedef fp16_t T_; constexpr int W_ = 32; CALL; } break;              \
+            default: { typedef fp16_t T_; constexpr int W_ = 64; CALL; } break;              \
+            }                                                                                \
+        }                                                                                    \
+    } while (0)
+
 static int check_batch(size_t M) {
     // include/network/SwiftNetMLP.h:293-300: the batch must be a multiple of 8
     if (M == 0 || (M % 8) != 0) return fail(TNN_ERR_INVALID_ARGUMENT, "batch size %zu is not a positive multiple of 8", M);
@@ -993,8 +894,8 @@ TNN_API int tnn_mlp_backward(const tnn_mlp_desc *desc, const void *d_prepared_bw
         return launch_backward128<fp16_t>(desc, d_prepared_bwd, d_dLdy, d_interm_fwd, deltas, d_interm_bwd != nullptr, d_dW, dW_is_fp32, d_dLdx, M,
                                           partials, s);
     }
-    TNN_DISPATCH_TW(desc, rc = (launch_backward<T_, W_>(desc, d_prepared_bwd, d_dLdy, d_interm_fwd, deltas, d_dLdx, M, s)));
+    TNN_DISPATCH_TW_UP_TO_64(desc, rc = (launch_backward<T_, W_>(desc, d_prepared_bwd, d_dLdy, d_interm_fwd, deltas, d_dLdx, M, s)));
     if (rc) return rc;
-    TNN_DISPATCH_TW(desc, rc = (launch_dw<T_, W_>(desc, deltas, d_interm_fwd, d_dW, dW_is_fp32, M, partials, s)));
+    TNN_DISPATCH_TW_UP_TO_64(desc, rc = (launch_dw<T_, W_>(desc, deltas, d_interm_fwd, d_dW, dW_is_fp32, M, partials, s)));
     return rc;
 }

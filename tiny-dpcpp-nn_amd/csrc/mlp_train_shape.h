@@ -16,7 +16,8 @@ template <int W> struct TrainShape {
     static size_t weight_bytes(int n_mats) { return (size_t)n_mats * NI * NK * 64 * 16; }
     static size_t lds_bytes(int n_mats) {
         const size_t stage = (size_t)WAVES * 2 * TILE_BYTES;
-        const size_t reduce = (size_t)n_mats * W * W * 4; // end-of-kernel sum over the waves that share a tile
+        // end-of-kernel sum over waves that each hold a whole dW: a tree that starts with four slots
+        const size_t reduce = SHARED ? 0 : (size_t)4 * n_mats * W * W * 4;
         const size_t main = 2 * weight_bytes(n_mats) + stage + 64; // + the arrival counters of the half-workgroups
         return main > reduce ? main : reduce;
     }

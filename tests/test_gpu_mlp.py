@@ -110,7 +110,7 @@ def test_activation_pairs_forward_backward(tnn, oracle, act, out_act):
 
 
 @pytest.mark.parametrize("dtype", [BF16, FP16])
-@pytest.mark.parametrize("W,n_hidden", [(16, 2), (32, 4), (128, 8), (64, 4)])
+@pytest.mark.parametrize("W,n_hidden", [(16, 2), (32, 4), (128, 8), (64, 4), (128, 3)])
 def test_backward_parity_widths(tnn, oracle, dtype, W, n_hidden):
     n_mats = n_hidden + 1
     M = 8 * 45

@@ -696,8 +696,8 @@ static int launch_backward128(const tnn_mlp_desc *d, const void *wprep_bwd, cons
     for (auto k : {k_top, k_mid})
         if (hipFuncSetAttribute(reinterpret_cast<const void *>(k), hipFuncAttributeMaxDynamicSharedMemorySize, (int)LayerBwd128::lds_bytes) != hipSuccess)
             return fail(TNN_ERR_HIP, "cannot reserve %zu bytes of LDS", LayerBwd128::lds_bytes);
-    if (hipFuncSetAttribute(reinterpret_cast<const void *>(k_pair), hipFuncAttributeMaxDynamicSharedMemorySize, (int)LayerBwd128::lds_bytes) != hipSuccess)
-        return fail(TNN_ERR_HIP, "cannot reserve %zu bytes of LDS", LayerBwd128::lds_bytes);
+    if (hipFuncSetAttribute(reinterpret_cast<const void *>(k_pair), hipFuncAttributeMaxDynamicSharedMemorySize, (int)LayerBwd128::pair_lds_bytes) != hipSuccess)
+        return fail(TNN_ERR_HIP, "cannot reserve %zu bytes of LDS", LayerBwd128::pair_lds_bytes);
     const T *fwd = static_cast<const T *>(interm_fwd);
     const T *input0 = x0 ? static_cast<const T *>(x0) : fwd; // the first matrix's input: the caller's x, or its copy in front of the activations
     T *dl = static_cast<T *>(deltas);
@@ -709,7 +709,7 @@ static int launch_backward128(const tnn_mlp_desc *d, const void *wprep_bwd, cons
         const bool top = (l == n_mats - 1);
         if (!top && l >= 1) {
             T *delta_out = l > 1 ? dl + (size_t)(l - 2) * mat : static_cast<T *>(dLdx);
-            TNN_LAUNCH(k_pair, dim3((unsigned)p.n_chunks), dim3(kLayerBwdThreads), LayerBwd128::lds_bytes, s, wb + (size_t)l * per_mat,
+            TNN_LAUNCH(k_pair, dim3((unsigned)p.n_chunks), dim3(kLayerBwdThreads), LayerBwd128::pair_lds_bytes, s, wb + (size_t)l * per_mat,
                        wb + (size_t)(l - 1) * per_mat, dl + (size_t)l * mat, fwd + (size_t)l * mat, l > 1 ? fwd + (size_t)(l - 1) * mat : input0,
                        keep_top_delta ? dl + (size_t)(l - 1) * mat : (T *)nullptr, delta_out, partials, n_mats, l, d->activation,
                        l > 1 ? d->activation : TNN_ACT_NONE, (long long)M, p.rows_per_chunk);

@@ -41,7 +41,7 @@ METRIC = "fused-MLP train & infer samples/s (w64, batch 2^18); % bf16 MFMA peak"
 # profiles/grid_forward_kernel.*.txt, profiles/grid_mlp_inference_kernel.*.txt and profiles/grid_backward_kernel.*.txt. Not measured live: counters need the profiler.
 MEASURED_TRAFFIC_BYTES = {
     ("train", 18): (55832.3 * 2.0 + 20488.0) * 1024,
-    ("infer", 18): (16786.6 * 2.0 + 32768.0) * 1024,
+    ("infer", 18): (16780.5 * 2.0 + 32795.7) * 1024,
     ("train_fb", 18): (98600.2 * 2.0 + 217143.4) * 1024,  # the backward kernel
     ("grid", 21): (6374561.8 * 2.0 + 132047.2) * 1024,           # points in the caller's order (--no-cell-order)
     ("grid_ordered", 21): (3584394.4 * 2.0 + 131865.3) * 1024,   # points in cell order, the default

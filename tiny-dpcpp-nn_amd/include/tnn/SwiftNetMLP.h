@@ -131,7 +131,7 @@ template <typename T, int WIDTH> class SwiftNetMLP : public Network<T> {
 
     static bool Supported(Activation a) { return a == Activation::ReLU || a == Activation::None || a == Activation::Sigmoid; }
 
-    void SanityCheck() const {
+    void SanityCheck() const override {
         static_assert(WIDTH == 16 || WIDTH == 32 || WIDTH == 64 || WIDTH == 128);
         static_assert(std::is_same<T, tnn::bf16>::value || std::is_same<T, tnn::half>::value);
         if (!Supported(m_activation)) throw std::runtime_error("m_activation must be ReLU or None or Sigmoid for now.");

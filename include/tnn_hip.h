@@ -4,9 +4,11 @@
  * the L2 loss, an Adam step, and the multi-resolution hash-grid encoding (forward / backward).
  *
  * Conventions
- *  - Every pointer named d_* is DEVICE memory owned by the caller. The library keeps no state,
- *    allocates nothing and is thread-safe; every call is asynchronous on `stream`
- *    (a hipStream_t passed as void*, NULL = the default stream).
+ *  - Every pointer named d_* is DEVICE memory owned by the caller. The library keeps no state between
+ *    calls, allocates nothing and is thread-safe; every call is asynchronous on `stream`
+ *    (a hipStream_t passed as void*, NULL = the default stream). Two exceptions, both stated where they
+ *    are declared: the process-wide limit set by tnn_debug_set_meeting_spin_limit (a testing aid), and the
+ *    fixed scratch array behind tnn_mlp_train_step_l2_static, which calls on one GPU share.
  *  - Return value: 0 on success, a negative tnn_status otherwise. No exception crosses this
  *    boundary; tnn_last_error() returns a thread-local message for the last failure.
  *  - "T" is the 2-byte storage type selected by tnn_mlp_desc::dtype (bf16 or fp16); all
@@ -75,6 +77,12 @@ int tnn_device_check(void);
 
 /* DeviceMatrix::fill / DeviceMatrices::fill (include/common/DeviceMatrix.h:167,381): n elements of dtype := value. */
 int tnn_fill(int dtype, void *d_ptr, size_t n, float value, tnn_stream_t stream);
+/* DeviceMatrix::fill_random (include/common/DeviceMatrix.h:169-178, the default table of a grid encoding: uniform in
+ * +-1e-4) and Network::initialize_xavier_normal (include/network/Network.h:271-295), both host generators plus a copy in
+ * the reference: element i := lo + (hi - lo) * u, u in [0, 1) with 24 random bits, a pure function of (seed,
+ * first_index + i) (the splitmix64 output function on seed + (first_index + i + 1) * 0x9E3779B97F4A7C15). The reference's
+ * sequences (oneMKL philox, std::random_device) are not reproducible; only the distribution is the same. */
+int tnn_fill_uniform(int dtype, void *d_ptr, size_t n, float lo, float hi, uint64_t seed, uint64_t first_index, tnn_stream_t stream);
 /* DeviceMatrix::copy_from_device / DeviceMem::copy_from_device (include/common/DeviceMatrix.h:198-201,
  * include/common/DeviceMem.h:91-95): element-wise type-converting copy (round to nearest even). */
 int tnn_cast(int dst_dtype, void *d_dst, int src_dtype, const void *d_src, size_t n, tnn_stream_t stream);
@@ -210,9 +218,11 @@ int tnn_mlp_train_step_l2_adam(const tnn_mlp_desc *desc, void *d_prepared_fwd, v
  * staged tiles meet at a counter in LDS; a wave waits there for at most `iterations` polls (default 2^22, far beyond any
  * real wait) so that a kernel always ends. A wave whose wait runs out marks its workgroup, and the call then delivers NaN
  * in the loss and in EVERY weight gradient (and, through Adam, in the weights) instead of a plausible wrong number.
- * Setting the limit to 0 forces that path from the host while every kernel still runs to its end. Returns the previous
- * limit; process-wide. */
-int tnn_debug_set_meeting_spin_limit(int iterations);
+ * Setting the limit to 0 forces that path from the host while every kernel still runs to its end.
+ * Returns a status (a negative limit is TNN_ERR_INVALID_ARGUMENT); *previous, when not NULL, receives the limit that was in
+ * force. The limit is process-wide and read at every launch: it is for single-threaded test programs only -- while it is
+ * lowered, every width-64 training or backward call of any thread of the process is affected. */
+int tnn_debug_set_meeting_spin_limit(int iterations, int *previous);
 
 /* tnn_mlp_train_step_l2 for callers that cannot allocate device memory: code recorded into a HIP graph, tight serving
  * loops, harnesses that forbid hipMalloc. It has no counterpart in the reference. It takes no workspace: the partial
@@ -344,8 +354,12 @@ int tnn_grid_mlp_inference_ordered(const tnn_grid_desc *grid, const tnn_mlp_desc
  * The encoding is evaluated inside the training kernel where tnn_mlp_train_step_l2_adam loads its input rows, so the
  * M x width encoded matrix is neither written nor read; dL/d(encoding) goes through the workspace into the scatter of
  * tnn_grid_backward (tnn_grid_backward_ordered when d_order is given). Same values as tnn_grid_forward (out_dtype = network
- * type, padded_width = width) + tnn_mlp_train_step_l2_adam (with d_dLdx) + tnn_grid_backward: network weights and loss bit
- * for bit, the table's gradient up to the order of its fp32 additions.
+ * type, padded_width = width) + tnn_mlp_train_step_l2_adam (with d_dLdx) + tnn_grid_backward. With d_x (the caller's order):
+ * outputs, loss, Adam state and re-staged weights bit for bit, the table's gradient up to the order of its fp32 additions
+ * (atomic sums, as in the reference). With d_order: every per-row result (d_y, dL/d(encoding)) is still bit-exact, but the
+ * place of a point among the points of its cell is taken with atomics when the order is built, so the tiles hold other rows
+ * from run to run and every sum over the batch (loss, weight gradients and what Adam makes of them, table gradient) is
+ * reproducible to fp32 rounding only, not bit for bit.
  *   d_x: M x n_dims fp32, or NULL when d_order holds the records of tnn_grid_order_points for the batch (rows of d_targets
  *   and d_y keep the caller's order either way). d_table: the encoding's parameters (param_dtype).
  *   d_grad_table: n_params fp32, overwritten or accumulated into as in tnn_grid_backward; it holds loss_scale x the gradient.

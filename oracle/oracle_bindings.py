@@ -64,6 +64,19 @@ class Oracle:
         self.L.tnn_oracle_round(_p(a), _p(out), a.size, dtype)
         return out
 
+    def splitmix64(self, seed, index):
+        self.L.tnn_oracle_splitmix64.restype = ctypes.c_uint64
+        self.L.tnn_oracle_splitmix64.argtypes = [ctypes.c_uint64, ctypes.c_uint64]
+        return int(self.L.tnn_oracle_splitmix64(seed, index))
+
+    def fill_uniform(self, n, lo, hi, seed, first_index, dtype):
+        out = np.empty(n, np.float32)
+        self.L.tnn_oracle_fill_uniform.restype = None
+        self.L.tnn_oracle_fill_uniform.argtypes = [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_float, ctypes.c_float, ctypes.c_uint64,
+                                                   ctypes.c_uint64, ctypes.c_int]
+        self.L.tnn_oracle_fill_uniform(_p(out), n, lo, hi, seed, first_index, dtype)
+        return out
+
     def num_threads(self):
         return self.L.tnn_oracle_num_threads()
 

@@ -26,8 +26,10 @@
  *   sh_forward .................. golden rows of test/python/test_encodings.py:389-573 (degree 4), the degree-1 vector of
  *                                 test/doctest_encodings.cpp:197-232, the reference's explicit expressions of bands 0-3
  *                                 (sh_explicit16) and of single members of bands 4-7, orthonormality on the sphere
+ *   fill_uniform ................ the library's own seeded generator (no counterpart sequence in the reference): the
+ *                                 published splitmix64 test vector, range, mean and variance of the uniform law
  *   default table init / Xavier init of the reference: parity unpinned (unseeded / closed-source
- *   generators in the reference); not restated here.
+ *   generators in the reference); their sequences are not restated here, only the distribution is matched.
  */
 #include <math.h>
 #ifndef M_PI
@@ -786,4 +788,23 @@ TNN_ORACLE_API int tnn_oracle_sh_forward(int degree, const float *xin, size_t M,
         for (int j = degree * degree; j < padded_width; ++j) row[j] = 1.0f;
     }
     return 0;
+}
+
+/* The library's seeded uniform fill (tnn_fill_uniform): stands where the reference draws from oneMKL philox
+ * (include/common/DeviceMatrix.h:169-178) and from std::mt19937(std::random_device) (include/network/Network.h:271-295).
+ * splitmix64 (Steele, Lea, Flood 2014; Vigna's public-domain splitmix64.c): state += gamma per draw, output = mix(state). */
+TNN_ORACLE_API uint64_t tnn_oracle_splitmix64(uint64_t seed, uint64_t index) {
+    uint64_t z = seed + (index + 1ull) * 0x9E3779B97F4A7C15ull;
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+    return z ^ (z >> 31);
+}
+
+TNN_ORACLE_API void tnn_oracle_fill_uniform(float *out, size_t n, float lo, float hi, uint64_t seed, uint64_t first_index, int dtype) {
+    const float span = hi - lo;
+    for (size_t i = 0; i < n; ++i) {
+        const float u = (float)(uint32_t)(tnn_oracle_splitmix64(seed, first_index + i) >> 40) * 5.9604644775390625e-8f;
+        const volatile float prod = span * u; /* two roundings, as the kernel */
+        out[i] = round_T(lo + prod, dtype);
+    }
 }

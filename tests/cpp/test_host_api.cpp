@@ -174,28 +174,41 @@ static void test_json() {
     CHECK(json::parse(j.dump())["n_levels"].get<int>() == 16);
 }
 
-// File helpers of io.h: what one writes the other reads back; formats as the reference's own files use them
-// (one value per line for weights, delimiter-separated rows for target vectors, binary PGM for images).
+// File helpers of io.h: what one writes the other reads back; number files as the reference's own tools write them (one value
+// per line) or comma-separated; malformed content and missing files are errors.
 static void test_io_files() {
     const std::string dir = "/tmp/tnn_io_test_";
-    const std::vector<float> values{0.5f, -1.25f, 3.0f, 1e-3f};
+    const std::vector<float> values{0.5f, -1.25f, 3.0f, 1e-3f, 0.1f, -3.4e38f};
     io::saveCSV(dir + "v.csv", values);
-    CHECK(io::loadCSV(dir + "v.csv") == values);
-    CHECK(io::loadVectorFromCSV<float>(dir + "v.csv") == values);
-    CHECK(io::loadCSV(dir + "missing.csv").empty());
+    CHECK(io::loadVectorFromCSV<float>(dir + "v.csv") == values); // max_digits10: bit-exact round trip
     CHECK(throws<std::invalid_argument>([&] { io::loadVectorFromCSV<float>(dir + "missing.csv"); }));
+    CHECK(throws<std::invalid_argument>([&] { io::saveCSV(std::string("/nonexistent-dir/v.csv"), values); }));
     {
         std::ofstream f(dir + "t.csv");
-        f << "1;2;3\n4.5;-6\n";
+        f << "1,2;3\r\n4.5, -6\n\n  7e-1\t8";
     }
-    const auto rows = io::readTargetVectorsFromFile(dir + "t.csv", ';');
-    CHECK(rows.size() == 2 && rows[0] == (std::vector<float>{1.f, 2.f, 3.f}) && rows[1] == (std::vector<float>{4.5f, -6.f}));
-    CHECK(io::readTargetVectorsFromFile(dir + "missing.csv", ',').empty());
-    const std::vector<unsigned char> image{0, 64, 128, 255, 1, 2};
-    io::saveImageToPGM(dir + "i.pgm", 3, 2, image);
-    std::ifstream f(dir + "i.pgm", std::ios::binary);
-    std::string bytes((std::istreambuf_iterator<char>(f)), std::istreambuf_iterator<char>());
-    CHECK(bytes == std::string("P5\n3 2\n255\n") + std::string(image.begin(), image.end()));
+    CHECK(io::loadVectorFromCSV<float>(dir + "t.csv") == (std::vector<float>{1.f, 2.f, 3.f, 4.5f, -6.f, 0.7f, 8.f}));
+    {
+        std::ofstream f(dir + "bad.csv");
+        f << "1\n2x\n3\n";
+    }
+    CHECK(throws<std::invalid_argument>([&] { io::loadVectorFromCSV<float>(dir + "bad.csv"); }, "byte 2"));
+    {
+        std::ofstream f(dir + "huge.csv");
+        f << "1e60\n";
+    }
+    CHECK(throws<std::out_of_range>([&] { io::loadVectorFromCSV<float>(dir + "huge.csv"); }));
+    {
+        std::ofstream f(dir + "empty.csv");
+    }
+    CHECK(io::loadVectorFromCSV<float>(dir + "empty.csv").empty());
+    {
+        std::ofstream f(dir + "cfg.json");
+        f << "{\"otype\": \"HashGrid\", \"type\": \"Tiled\", \"interpolation\": \"Smoothstep\", \"n_levels\": 4}";
+    }
+    const json cfg = io::loadJsonConfig(dir + "cfg.json");
+    CHECK(cfg["type"].get<GridType>() == GridType::Tiled && cfg["interpolation"].get<InterpolationType>() == InterpolationType::Smoothstep);
+    CHECK(throws<std::runtime_error>([&] { io::loadJsonConfig(dir + "missing.json"); }, "Unable to open"));
     // unpacked [in][out] matrices, one value per line -> the packed parameter vector of a width-16 network
     std::vector<float> w(2 * 16 * 16);
     for (size_t i = 0; i < w.size(); ++i) w[i] = (float)(i % 97) / 128.0f;
@@ -207,6 +220,7 @@ static void test_io_files() {
         for (int k = 0; k < 16; ++k)
             for (int n = 0; n < 16; ++n) same = same && (float)packed[m * 256 + toPackedLayoutCoord(k * 16 + n, 16, 16)] == w[m * 256 + k * 16 + n];
     CHECK(same);
+    CHECK(throws<std::invalid_argument>([&] { (void)io::load_weights_as_packed_from_file<tnn::half, 16>(dir + "w.csv", 2, 16, 16); }, "the network has 768"));
 }
 
 // ------------------------------------------------------------------------------------------- GPU cases
@@ -362,7 +376,7 @@ static void test_swiftnet_errors() {
     using bf = tnn::bf16;
     CHECK(throws<std::runtime_error>([&] { SwiftNetMLP<bf, 64> n(q, 65, 64, 2, Activation::ReLU, Activation::None); }, "Input width of 128"));
     CHECK(throws<std::runtime_error>([&] { SwiftNetMLP<bf, 64> n(q, 64, 200, 2, Activation::ReLU, Activation::None); }, "not supported"));
-    CHECK(throws<std::invalid_argument>([&] { SwiftNetMLP<bf, 64> n(q, 0, 64, 2, Activation::ReLU, Activation::None); }, "width <= 0"));
+    CHECK(throws<std::invalid_argument>([&] { SwiftNetMLP<bf, 64> n(q, 0, 64, 2, Activation::ReLU, Activation::None); }, "width <= 0 cannot be padded"));
     CHECK(throws<std::runtime_error>([&] { SwiftNetMLP<bf, 64> n(q, 64, 64, 0, Activation::ReLU, Activation::None); }, "must be >= 1"));
     CHECK(throws<std::invalid_argument>([&] { SwiftNetMLP<bf, 64> n(q, 64, 64, -1, Activation::ReLU, Activation::None); }, "non-negative"));
     CHECK(throws<std::runtime_error>([&] { SwiftNetMLP<bf, 64> n(q, 64, 64, 2, Activation::Tanh, Activation::None); }, "m_activation must be"));

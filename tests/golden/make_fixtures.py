@@ -17,6 +17,31 @@ def numbers_between(text, start_marker, end_marker):
     return [float(t) for t in re.findall(r"-?\d+\.?\d*(?:[eE]-?\d+)?", text[s:e])]
 
 
+def polynomial_value(text, variables):
+    """Value of an arithmetic expression taken from the reference's source text. The text is parsed, never executed: only
+    numbers, the given variable names, unary +/- and the operators + - * / are accepted; anything else raises."""
+    import ast
+    import operator
+
+    binary = {ast.Add: operator.add, ast.Sub: operator.sub, ast.Mult: operator.mul, ast.Div: operator.truediv}
+    unary = {ast.UAdd: operator.pos, ast.USub: operator.neg}
+
+    def value(node):
+        if isinstance(node, ast.Expression):
+            return value(node.body)
+        if isinstance(node, ast.Constant) and type(node.value) in (int, float):
+            return float(node.value)
+        if isinstance(node, ast.Name) and node.id in variables:
+            return variables[node.id]
+        if isinstance(node, ast.BinOp) and type(node.op) in binary:
+            return binary[type(node.op)](value(node.left), value(node.right))
+        if isinstance(node, ast.UnaryOp) and type(node.op) in unary:
+            return unary[type(node.op)](value(node.operand))
+        raise ValueError(f"not a polynomial in {sorted(variables)}: {ast.dump(node)[:80]}")
+
+    return value(ast.parse(text, mode="eval"))
+
+
 def main():
     # test/doctest_packing.cpp:21-46 : get_packed_weights of the vector 1..512 (two 16x16 matrices)
     txt = open(os.path.join(REF, "test/doctest_packing.cpp")).read()
@@ -97,7 +122,7 @@ def main():
         env = dict(x=x, y=y, z=z, xy=x * y, xz=x * z, yz=y * z, x2=x * x, y2=y * y, z2=z * z)
         env.update(x4=env["x2"] ** 2, y4=env["y2"] ** 2, z4=env["z2"] ** 2)
         env.update(x6=env["x4"] * env["x2"], y6=env["y4"] * env["y2"], z6=env["z4"] * env["z2"])
-        expected.append([eval(e, {"__builtins__": {}}, env) for e in exprs])
+        expected.append([polynomial_value(e, env) for e in exprs])
     json.dump(
         {
             "source": "include/common/common_device.h:33-206 (the polynomials of sh_enc, evaluated in double precision)",

@@ -109,6 +109,8 @@ CASES = [
     (3, 16, 15, 16, 1.447, FP16, FP16, 3, 2048 * 9, "none"),  # config 5's shape, several rounds per wave
     (3, 12, 14, 8, 1.6, FP32, BF16, 4, 3000 * 8, "relu"),  # fp32 table, bf16 network, deepest supported, 24 of 32 pieces real
     (2, 5, 12, 16, 2.0, FP32, BF16, 1, 8, "sigmoid"),     # one tile of 8 rows, a piece that is half real
+    (2, 32, 10, 4, 1.2, FP16, FP16, 2, 4096, "none"),     # 32 levels: every column of the width-64 input is an encoded feature
+    (3, 27, 11, 4, 1.25, FP32, BF16, 3, 2056, "none"),    # more than 22 levels, last piece not full
 ]
 
 

@@ -27,6 +27,24 @@ def test_l2_loss(tnn, oracle, dtype, tdt):
     assert np.allclose(tnn.host(grads), 4.0 * 2 * 0.375 / 128, rtol=4e-3)
 
 
+@pytest.mark.parametrize("dtype", [BF16, FP16, FP32])
+def test_fill_uniform(tnn, oracle, dtype):
+    """The seeded initialiser (default grid table, Xavier weights) equals the oracle's restatement bit for bit, whatever the
+    size of the launch, and an offset into the sequence continues it."""
+    from tiny_dpcpp_nn import _lib
+    from tiny_dpcpp_nn.cabi import ptr
+    for n, lo, hi, seed, first in ((1, -1.0, 1.0, 0, 0), (100003, -1e-4, 1e-4, 777, 0), (1 << 22, -0.2165, 0.2165, 2 ** 63 + 5, 2 ** 40)):
+        t = tnn.empty((n,), dtype, fill=float("nan"))
+        _lib.check(tnn.lib.tnn_fill_uniform(dtype, ptr(t), n, lo, hi, seed, first, tnn.stream()))
+        assert np.array_equal(tnn.host(t), oracle.fill_uniform(n, lo, hi, seed, first, dtype))
+    a, b = tnn.empty((1000,), FP32), tnn.empty((400,), FP32)
+    _lib.check(tnn.lib.tnn_fill_uniform(FP32, ptr(a), 1000, 0.0, 1.0, 3, 0, tnn.stream()))
+    _lib.check(tnn.lib.tnn_fill_uniform(FP32, ptr(b), 400, 0.0, 1.0, 3, 600, tnn.stream()))
+    assert torch.equal(a[600:], b)
+    assert tnn.lib.tnn_fill_uniform(FP32, ptr(a), 10, 1.0, 0.0, 3, 0, tnn.stream()) == _lib.TNN_ERR_INVALID_ARGUMENT
+    assert tnn.lib.tnn_fill_uniform(7, ptr(a), 10, 0.0, 1.0, 3, 0, tnn.stream()) == _lib.TNN_ERR_UNSUPPORTED
+
+
 def test_adam(tnn, oracle):
     rng = np.random.default_rng(1)
     n = 20480
@@ -245,7 +263,10 @@ def test_a_meeting_that_gives_up_poisons_the_step(tnn, oracle):
     tt = torch.from_numpy(rng.uniform(0, 1, (M, W)).astype(np.float32)).to(tnn.dev)
     good = tnn.train_step_l2(desc, pf, pb, xt, tt, 1.0)
     torch.cuda.synchronize()
-    old = tnn.lib.tnn_debug_set_meeting_spin_limit(0)
+    import ctypes
+    before = ctypes.c_int(-1)
+    assert tnn.lib.tnn_debug_set_meeting_spin_limit(0, ctypes.byref(before)) == _lib.TNN_OK
+    old = before.value
     try:
         assert old == 1 << 22
         y, loss, dW, dX = tnn.train_step_l2(desc, pf, pb, xt, tt, 1.0)
@@ -254,7 +275,7 @@ def test_a_meeting_that_gives_up_poisons_the_step(tnn, oracle):
         _, dW_b, dX_b = tnn.backward(desc, pb, g, interm, dw_fp32=True)
         torch.cuda.synchronize()
     finally:
-        assert tnn.lib.tnn_debug_set_meeting_spin_limit(old) == 0
+        assert tnn.lib.tnn_debug_set_meeting_spin_limit(old, ctypes.byref(before)) == _lib.TNN_OK and before.value == 0
     assert torch.isnan(loss).all() and torch.isnan(dW).all(), "a step whose waits gave up must not return numbers"
     assert torch.isnan(dW_b).all()
     # what does not depend on other waves' tiles is still right
@@ -263,4 +284,5 @@ def test_a_meeting_that_gives_up_poisons_the_step(tnn, oracle):
     torch.cuda.synchronize()
     for a, b in zip(again, good):
         assert torch.equal(a.view(torch.uint8), b.view(torch.uint8))
-    assert tnn.lib.tnn_debug_set_meeting_spin_limit(-1) == _lib.TNN_ERR_INVALID_ARGUMENT
+    assert tnn.lib.tnn_debug_set_meeting_spin_limit(-1, None) == _lib.TNN_ERR_INVALID_ARGUMENT
+    assert tnn.lib.tnn_debug_set_meeting_spin_limit(1 << 22, ctypes.byref(before)) == _lib.TNN_OK and before.value == 1 << 22

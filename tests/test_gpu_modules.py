@@ -384,11 +384,79 @@ def test_network_with_grid_encoding_fused_inference(tcnn, dtype, n_dims, grid, b
         sh.network.tnn_module.inference_with_encoding(sh.encoding.tnn_module, torch.rand((8, 3), device=DEVICE))
 
 
+class SimpleSGD(torch.optim.Optimizer):
+    """The reference's debugging optimizer (test/python/test_training.py:28-51): it updates through `p.data`, which PyTorch's
+    version counter does not see."""
+
+    def __init__(self, params, lr):
+        super().__init__(params, dict(lr=lr))
+
+    def step(self, closure=None):
+        for group in self.param_groups:
+            for p in group["params"]:
+                if p.grad is not None:
+                    p.data.copy_(p.data - group["lr"] * p.grad.data)
+
+
+def test_training_through_data_writes(tcnn):
+    """The reference's SimpleSGDOptimizer loop (test/python/test_training.py:28-51, 62-140): every step writes the parameters
+    through `.data`; the next forward must run on the new weights, so the loss of a linear regression target falls."""
+    torch.manual_seed(5)
+    width = 32
+    net = tcnn.Network(width, 1, net_config(width, 2, "relu", "none"), dtype=torch.bfloat16)
+    opt = SimpleSGD(net.parameters(), lr=1e-2)
+    x = torch.ones((8, width), device=DEVICE)
+    target = 0.5 * x[:, :1]
+    net.train()
+    losses, outputs = [], []
+    for _ in range(40):
+        y = net(x)
+        loss = (y.float() - target).square().mean()
+        opt.zero_grad()
+        loss.backward()
+        opt.step()
+        losses.append(float(loss))
+        outputs.append(y.detach().clone())
+    assert not torch.equal(outputs[0], outputs[1]), "a step written through .data did not reach the kernels"
+    assert losses[-1] < 0.05 * losses[0], losses
+
+
+def test_params_data_assignment_reaches_the_kernels(tcnn):
+    """`network.params.data[:] = ...` followed by a forward (test/python/test_padding_bias.py:169-172), in evaluation mode too."""
+    torch.manual_seed(6)
+    net = tcnn.Network(8, 4, net_config(32, 2, "none", "none"), dtype=torch.bfloat16, use_bias=False)
+    x = torch.rand((16, 8), device=DEVICE)
+    for train in (True, False):
+        net.train(train)
+        net.params.data[:] = 0.0
+        with torch.no_grad():
+            assert float(net(x).float().abs().max()) == 0.0
+        net.params.data[:] = torch.full_like(net.params, 0.03125)
+        with torch.no_grad():
+            y = net(x)
+        # every weight 1/32, no activation: column sums of x over the 8 real inputs, then 32 * (1/32) per later matrix
+        expect = (x.to(torch.bfloat16).float().sum(1, keepdim=True) / 32).expand(-1, 4)
+        assert torch.allclose(y.float(), expect, rtol=2e-2, atol=1e-3)
+    # the fused encoding + network route reads both modules' parameters the same way
+    nwe = tcnn.NetworkWithInputEncoding(2, 3, net_config(64, 2), dict(GRID_2D), dtype=torch.float16)
+    nwe.eval()
+    pts = torch.rand((64, 2), device=DEVICE)
+    with torch.no_grad():
+        nwe.encoding.params.data[:] = torch.rand_like(nwe.encoding.params) * 2 - 1
+        y0 = nwe(pts).clone()
+        nwe.encoding.params.data[:] = 0.0
+        y1 = nwe(pts)
+    assert float(y0.float().abs().max()) > 0.0 and float(y1.float().abs().max()) == 0.0
+
+
 def test_parameters_are_pushed_when_they_change(tcnn):
-    """forward() refreshes the native module's copy of the parameters when `params` changed since the last push: an
-    optimizer step, copy_() and a replaced Parameter are all seen; a write through `.data` needs an explicit set_params()."""
+    """With push_params_every_forward switched off, forward() refreshes the native module's copy of the parameters only when
+    `params` changed since the last push: an optimizer step, copy_() and a replaced Parameter are all seen; a write through
+    `.data` then needs an explicit set_params(). The default pushes every time, as the reference does."""
     torch.manual_seed(11)
     net = tcnn.Network(8, 4, net_config(32, 2), dtype=torch.bfloat16)
+    assert net.push_params_every_forward
+    net.push_params_every_forward = False
     x = torch.rand((64, 8), device=DEVICE)
     opt = torch.optim.Adam(net.parameters(), lr=1e-2)
     net.train()

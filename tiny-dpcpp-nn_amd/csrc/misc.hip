@@ -115,6 +115,20 @@ template <typename T> __global__ void fill_kernel(T *__restrict__ p, size_t n, T
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) p[i] = v;
 }
 
+// Element i := lo + (hi - lo) * u_i, where u_i in [0, 1) is the top 24 bits of the splitmix64 output for the state
+// seed + (first + i + 1) * 0x9E3779B97F4A7C15: the value depends on (seed, first + i) only, not on the launch shape.
+template <typename T> __global__ void fill_uniform_kernel(T *__restrict__ p, size_t n, float lo, float hi, unsigned long long seed, unsigned long long first) {
+    const float span = hi - lo;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
+        unsigned long long z = seed + (first + i + 1ull) * 0x9E3779B97F4A7C15ull;
+        z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+        z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+        z ^= z >> 31;
+        const float u = (float)(unsigned int)(z >> 40) * 5.9604644775390625e-8f; // 2^-24: exact
+        p[i] = (T)as_fp32(lo + as_fp32(span * u));
+    }
+}
+
 template <typename D, typename S> __global__ void cast_kernel(D *__restrict__ d, const S *__restrict__ s, size_t n) {
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) d[i] = (D)(float)s[i];
 }
@@ -279,6 +293,23 @@ TNN_API int tnn_fill(int dtype, void *d_ptr, size_t n, float value, tnn_stream_t
     default: return fail(TNN_ERR_UNSUPPORTED, "dtype %d", dtype);
     }
     return check_launch("fill_kernel");
+}
+
+TNN_API int tnn_fill_uniform(int dtype, void *d_ptr, size_t n, float lo, float hi, uint64_t seed, uint64_t first_index, tnn_stream_t stream) {
+    if (!d_ptr && n) return fail(TNN_ERR_INVALID_ARGUMENT, "NULL pointer argument");
+    if (!(lo <= hi)) return fail(TNN_ERR_INVALID_ARGUMENT, "tnn_fill_uniform: bounds %g, %g", (double)lo, (double)hi);
+    if (n == 0) return TNN_OK;
+    size_t blocks = (n + 255) / 256;
+    if (blocks > 8192) blocks = 8192;
+    hipStream_t s = as_stream(stream);
+    const unsigned long long sd = seed, fi = first_index;
+    switch (dtype) {
+    case TNN_BF16: TNN_LAUNCH((fill_uniform_kernel<bf16_t>), dim3((unsigned)blocks), dim3(256), 0, s, (bf16_t *)d_ptr, n, lo, hi, sd, fi); break;
+    case TNN_FP16: TNN_LAUNCH((fill_uniform_kernel<fp16_t>), dim3((unsigned)blocks), dim3(256), 0, s, (fp16_t *)d_ptr, n, lo, hi, sd, fi); break;
+    case TNN_FP32: TNN_LAUNCH((fill_uniform_kernel<float>), dim3((unsigned)blocks), dim3(256), 0, s, (float *)d_ptr, n, lo, hi, sd, fi); break;
+    default: return fail(TNN_ERR_UNSUPPORTED, "dtype %d", dtype);
+    }
+    return check_launch("fill_uniform_kernel");
 }
 
 template <typename D> static int launch_cast(D *d, int src_dtype, const void *src, size_t n, hipStream_t s) {

@@ -77,7 +77,9 @@ size_t fused_train_workspace_bytes(const tnn_mlp_desc *d, size_t M) {
 
 } // namespace tnn
 
-TNN_API int tnn_debug_set_meeting_spin_limit(int iterations) {
+TNN_API int tnn_debug_set_meeting_spin_limit(int iterations, int *previous) {
     if (iterations < 0) return tnn::fail(TNN_ERR_INVALID_ARGUMENT, "the spin limit cannot be negative");
-    return tnn::g_meeting_spin_limit.exchange(iterations, std::memory_order_relaxed);
+    const int before = tnn::g_meeting_spin_limit.exchange(iterations, std::memory_order_relaxed);
+    if (previous) *previous = before;
+    return TNN_OK;
 }

@@ -13,12 +13,13 @@ template <int W> struct TrainShape {
     static constexpr int PITCH = W * 2 + 16;       // bytes per staged row (16-byte skew)
     static constexpr int TILE_BYTES = 32 * PITCH;
     static constexpr int WAVES = kTrainThreads / 64;
+    static constexpr int CONTROL_BYTES = 64; // behind the staged tiles: the groups' arrival counters and the gave-up flag
     static size_t weight_bytes(int n_mats) { return (size_t)n_mats * NI * NK * 64 * 16; }
     static size_t lds_bytes(int n_mats) {
         const size_t stage = (size_t)WAVES * 2 * TILE_BYTES;
         // end-of-kernel sum over waves that each hold a whole dW: a tree that starts with four slots
         const size_t reduce = SHARED ? 0 : (size_t)4 * n_mats * W * W * 4;
-        const size_t main = 2 * weight_bytes(n_mats) + stage + 64; // + the arrival counters of the half-workgroups
+        const size_t main = 2 * weight_bytes(n_mats) + stage + CONTROL_BYTES;
         return main > reduce ? main : reduce;
     }
 };

@@ -107,17 +107,11 @@ template <typename T, MatrixLayout _layout = MatrixLayout::RowMajor> class Devic
         tnn::abi_check(tnn_fill(tnn::dtype_of<T>::value, m_data, n_elements(), (float)val, m_q.abi()));
         return tnn::event(m_q.get());
     }
-    // Uniform values in [lower, upper) from a fixed seed (the reference uses oneMKL philox with seed 777; the
-    // sequence itself is not reproduced, only the distribution).
+    // Uniform values in [lower, upper), drawn on the device from a fixed seed (the reference draws from oneMKL philox with
+    // seed 777, DeviceMatrix.h:169-178 there; that sequence is not reproducible, the distribution is the same).
     tnn::event fill_random(const T lower_bound, const T upper_bound) {
-        std::vector<T> h(n_elements());
-        uint64_t state = 777;
-        const float lo = (float)lower_bound, hi = (float)upper_bound;
-        for (auto &v : h) {
-            state = state * 6364136223846793005ull + 1442695040888963407ull;
-            v = T(lo + (hi - lo) * (float)((state >> 40) * (1.0 / 16777216.0)));
-        }
-        return copy_from_host(h);
+        tnn::abi_check(tnn_fill_uniform(tnn::dtype_of<T>::value, m_data, n_elements(), (float)lower_bound, (float)upper_bound, 777, 0, m_q.abi()));
+        return tnn::event(m_q.get());
     }
     tnn::event copy_to_host(std::vector<T> &out) const {
         if (out.size() < n_elements()) throw std::invalid_argument("Target too small.");

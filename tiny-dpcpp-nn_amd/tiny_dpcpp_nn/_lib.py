@@ -62,6 +62,7 @@ SIGNATURES = {
     "tnn_abi_version": (c_int, []),
     "tnn_device_check": (c_int, []),
     "tnn_fill": (c_int, [c_int, c_void_p, c_size_t, c_float, c_void_p]),
+    "tnn_fill_uniform": (c_int, [c_int, c_void_p, c_size_t, c_float, c_float, ctypes.c_uint64, ctypes.c_uint64, c_void_p]),
     "tnn_cast": (c_int, [c_int, c_void_p, c_int, c_void_p, c_size_t, c_void_p]),
     "tnn_pack_weights": (c_int, [c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]),
     "tnn_unpack_weights": (c_int, [c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]),
@@ -84,7 +85,7 @@ SIGNATURES = {
         [POINTER(MlpDesc), c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
          c_size_t, c_void_p, c_size_t, c_void_p],
     ),
-    "tnn_debug_set_meeting_spin_limit": (c_int, [c_int]),
+    "tnn_debug_set_meeting_spin_limit": (c_int, [c_int, ctypes.POINTER(c_int)]),
     "tnn_mlp_train_step_l2_static_max_bytes": (c_size_t, []),
     "tnn_mlp_train_step_l2_static": (
         c_int,

@@ -8,9 +8,12 @@ filled with ones when `use_bias` and zeros otherwise), the same loss scaling (12
 layout conventions (`params` of a network is the packed layout, `set_params(tensor)` takes unpacked matrices). The device
 is PyTorch-ROCm's "cuda" where the reference has "xpu".
 
-Differences in behaviour, all of them savings: the native module's copy of the parameters is refreshed when `params` has
-changed since it was last pushed (PyTorch's version counter), not on every forward; and in evaluation mode under
-`torch.no_grad()` a grid encoding and its network run as one kernel.
+As in the reference (modules.py:253), every forward pushes `params` to the native module first, so that any way of
+writing them is seen, `params.data[...] = ...` included. The push is one small kernel on the device. A caller that only
+ever updates `params` through operations PyTorch's version counter sees (optimizers, copy_(), load_state_dict) can switch
+the push off for unchanged parameters with `module.push_params_every_forward = False`.
+
+One difference in behaviour, a saving: a grid encoding and its network run as one kernel, in evaluation and in training.
 
 All compute goes through the extension module `tiny_dpcpp_nn_pybind_module` (HIP kernels); importing this file fails if it
 is not built. There is no PyTorch fallback.
@@ -129,6 +132,10 @@ class Module(torch.nn.Module):
         self.use_bias = use_bias
         self.store_params_as_full_precision = store_params_as_full_precision
         self.loss_scale = 128.0 if dtype == torch.float16 else 1.0
+        # True (the reference's behaviour): every forward pushes `params` first. False: only when the tensor's identity, storage
+        # address or version counter changed since the last push -- a write through `.data` changes none of them and then
+        # needs an explicit set_params().
+        self.push_params_every_forward = True
         self._pushed = None  # (tensor identity, storage address, version) of `params` when the native module last took it
         if not init_module:
             return
@@ -163,7 +170,7 @@ class Module(torch.nn.Module):
     def set_params(self, params=None):
         """`params` given: a flat tensor of unpacked [in][out] matrices (network) or the table (encoding); it is pushed to the
         native module and `self.params` takes what the module then holds. `None`: push `self.params` as it is (a network's is
-        already packed). Always pushes; `forward` only does so when `params` has changed."""
+        already packed)."""
         if self.tnn_module.n_params() == 0:
             if params is not None:
                 raise RuntimeError("Network has no parameters. Cannot set params")
@@ -177,10 +184,11 @@ class Module(torch.nn.Module):
                 self.params.copy_(self.get_params().reshape(self.params.shape))
         self._pushed = self._params_state()
 
-    def _push_if_changed(self):
-        """In-place updates (optimizer steps, copy_, load_state_dict) raise the tensor's version; a replaced tensor has another
-        identity or address. Writes through `.data` do neither: call set_params() after those."""
-        if self.tnn_module.n_params() and self._pushed != self._params_state():
+    def _push_before_forward(self):
+        """What the reference does in front of every forward (modules.py:253): set_params(). With push_params_every_forward
+        switched off, only when `params` is known to have changed: in-place updates (optimizer steps, copy_, load_state_dict)
+        raise the tensor's version and a replaced tensor has another identity or address; writes through `.data` do neither."""
+        if self.tnn_module.n_params() and (self.push_params_every_forward or self._pushed != self._params_state()):
             self.set_params()
 
     def get_params(self):
@@ -193,7 +201,7 @@ class Module(torch.nn.Module):
 
     def forward(self, x):
         batch = x.shape[0]
-        self._push_if_changed()
+        self._push_before_forward()
         y = _NativeCall.apply(self, self._prepare_input(x).contiguous(), self.params)
         return y[:batch]
 
@@ -296,8 +304,8 @@ class NetworkWithInputEncoding(Module):
         of the two modules in turn (the reference's only route)."""
         batch = x.shape[0]
         rows = _rows_padded(batch)
-        self.encoding._push_if_changed()
-        self.network._push_if_changed()
+        self.encoding._push_before_forward()
+        self.network._push_before_forward()
         positions = _pad_rows(x, rows).to(torch.float32).contiguous()
         y = self.network.tnn_module.inference_with_encoding(self.encoding.tnn_module, positions)
         return y.reshape(rows, -1)[:batch, : self.n_output_dims]

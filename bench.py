@@ -43,8 +43,8 @@ MEASURED_TRAFFIC_BYTES = {
     ("train", 18): (55832.3 * 2.0 + 20488.0) * 1024,
     ("infer", 18): (16780.5 * 2.0 + 32795.7) * 1024,
     ("train_fb", 18): (98600.2 * 2.0 + 217143.4) * 1024,  # the backward kernel
-    ("grid", 21): (6374561.8 * 2.0 + 132047.2) * 1024,           # points in the caller's order (--no-cell-order)
-    ("grid_ordered", 21): (3584394.4 * 2.0 + 131865.3) * 1024,   # points in cell order, the default
+    ("grid", 21): (6380144.1 * 2.0 + 132091.7) * 1024,           # points in the caller's order (--no-cell-order)
+    ("grid_ordered", 21): (3576886.7 * 2.0 + 131888.5) * 1024,   # points in cell order, the default
     ("grid_mlp", 21): (6610053.5 * 2.0 + 263715.5) * 1024,
     ("grid_mlp_ordered", 21): (3915783.4 * 2.0 + 264728.9) * 1024,
     ("grid_train", 18): (108943.2 * 2.0 + 236762.7) * 1024,  # the scatter kernel; an atomic request counts as a 32-byte write
@@ -304,13 +304,13 @@ class Bench:
         # fp32 master weights in the packed parameter layout, as the reference's Python module keeps them
         master = t.pack(FP32, W, n_mats, torch.from_numpy(w.reshape(-1)).to(t.dev))
         pf, pb = t.prepare_packed(desc, master, src_is_fp32=True)
-        return dict(W=W, n_hidden=n_hidden, n_mats=n_mats, M=M, desc=desc, w=w, gen=gen, x=x, master=master, pf=pf, pb=pb)
+        return dict(W=W, n_hidden=n_hidden, n_mats=n_mats, M=M, desc=desc, w=w, gen=gen, x=x, master=master, master0=master.clone(), pf=pf, pb=pb)
 
     def parity_mlp(self, c, targets):
         """One training step and one inference on the tensors that are timed, against the oracle. Returns the differences."""
         np, torch, t, oracle, lib = self.np, self.torch, self.t, self.oracle, self.lib
         from tiny_dpcpp_nn.cabi import ptr
-        from tolerances import BF16, assert_propagated, max_norm_rel
+        from tolerances import BF16, PROPAGATED, assert_close, assert_propagated, bar_report, max_norm_rel
         W, n_mats, M, desc = c["W"], c["n_mats"], c["M"], c["desc"]
         w_T = oracle.round(c["w"], BF16)  # the weights as the kernels see them
         xh, th = t.host(c["x"]), targets.cpu().numpy()
@@ -319,14 +319,24 @@ class Bench:
         y_inf = t.host(t.inference(desc, c["pf"], c["x"]))
         assert_propagated(y_inf, interm[-1], BF16, "bench parity: inference output")
         res["infer_output_max_norm_rel"] = max_norm_rel(y_inf, interm[-1])
-        y, loss, dW, _ = t.train_step_l2(desc, c["pf"], c["pb"], c["x"], targets, 1.0, want_dx=False)
+        c["y_inference_checked"] = y_inf  # the sub-batch and rotating inference legs compare their rows with these bits
+        y, loss, dW, dX = t.train_step_l2(desc, c["pf"], c["pb"], c["x"], targets, 1.0, want_dx=True)
         yh = t.host(y)
         assert_propagated(yh, interm[-1], BF16, "bench parity: training-step output")
         values, grads = oracle.l2_loss(BF16, yh, th, 1.0)
         ref_loss = float(values.astype(np.float64).sum())
         assert abs(float(loss.item()) - ref_loss) <= 1e-4 * ref_loss, "bench parity: loss"
-        _, rdW, _ = oracle.mlp_backward_T(BF16, W, n_mats, "relu", "none", w_T, interm, grads, want_dx=False, round_dw=False)
-        dWh = t.host(dW)
+        _, rdW, rdX = oracle.mlp_backward_T(BF16, W, n_mats, "relu", "none", w_T, interm, grads, want_dx=True, round_dw=False)
+        dWh, dXh = t.host(dW), t.host(dX)
+        # dL/dx is a per-row quantity of natural size 1/M (dL/dy = 2 (y - t) / (M W)); a row whose ReLU mask flipped on a rounding
+        # boundary differs in all its elements and is outside any max-norm bound, so the elementwise bar is the check here
+        dx_scale = 1.0 / M
+        assert_close(dXh, rdX, BF16, "bench parity: dL/dx", scale=dx_scale, frac_ok=PROPAGATED)
+        # where the results stand against the STRICT elementwise bar (the end-to-end checks above allow 0.2 % of the elements
+        # outside it, none beyond 4x): the counts that actually leave it at this size
+        res["strict_bar"] = {"y": bar_report(yh, interm[-1], BF16), "dW": bar_report(dWh, rdW, BF16, scale=float(np.abs(rdW).max())),
+                             "dLdx": bar_report(dXh, rdX, BF16, scale=dx_scale)}
+        res["dLdx_max_norm_rel"] = max_norm_rel(dXh, rdX)
         res["dW_max_norm_rel"] = max(max_norm_rel(dWh[l], rdW[l]) for l in range(n_mats))
         assert res["dW_max_norm_rel"] < 1e-2, "bench parity: dW"
         assert_propagated(dWh, rdW, BF16, "bench parity: dW", scale=float(np.abs(rdW).max()))
@@ -360,9 +370,11 @@ class Bench:
         a = (ptr(pf), ptr(pb), ptr(c["x"]), ptr(targets), ptr(loss), ptr(master), ptr(m), ptr(v), ptr(ws))
         hip = HipEvents()
 
-        def step(i, mid=None):
+        dLdx = torch.empty_like(c["x"])
+
+        def step(i, mid=None, dx=None):
             rc = lib.tnn_mlp_train_step_l2_adam(d, a[0], a[1], a[2], a[3], 1.0, None, a[4], a[5], a[6], a[7], i + 1, 1e-3, 0.9, 0.99, 1e-15,
-                                                None, None, M, a[8], ws_bytes, mid, s)
+                                                None, dx, M, a[8], ws_bytes, mid, s)
             if rc:
                 raise RuntimeError(lib.tnn_last_error())
 
@@ -377,47 +389,91 @@ class Bench:
         nk = 50
         ks, ke = [hip.create() for _ in range(nk)], [hip.create() for _ in range(nk)]
 
+        # ... and the same once more with dL/dx requested (one more product per tile and a batch-sized store)
+        kxs, kxe = [hip.create() for _ in range(nk)], [hip.create() for _ in range(nk)]
+        xs = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
+
         def bracketed():
             for i in range(nk):
                 hip.record(ks[i], s)
                 step(timer.n + i, ke[i])
+            for i in range(nk):
+                hip.record(kxs[i], s)
+                step(timer.n + nk + i, kxe[i], ptr(dLdx))
+            xs[0].record()
+            for i in range(self.K):
+                step(timer.n + 2 * nk + i, None, ptr(dLdx))
+            xs[1].record()
 
         tm = timer.run(step, tail=bracketed)
         kern_ms = statistics.median(hip.elapsed_ms(x, y) for x, y in zip(ks, ke))
-        flops = 3 * 2 * M * W * W * n_mats  # reference convention: forward + backward-data + dW
+        kern_dx_ms = statistics.median(hip.elapsed_ms(x, y) for x, y in zip(kxs, kxe))
+        step_dx_ms = xs[0].elapsed_time(xs[1]) / self.K
+        # Reference convention (benchmarks/common_benchmarks.h:119-121): forward + backward-data + dW = 3 products per matrix,
+        # whether or not dL/dinput is formed. The timed step passes no dL/dx buffer (Trainer::training_step does not either),
+        # so the kernel executes 3 * n_mats - 1 of those products; both fractions are given.
+        flops = 3 * 2 * M * W * W * n_mats
+        executed = (3 * n_mats - 1) * 2 * M * W * W
         lg = int(np.log2(M))
         ach = flops / (kern_ms * 1e-3) / 1e12
         roof = {"bound": "mfma", "achieved": ach, "peak": PEAK_MFMA_BF16, "unit": "TFLOP/s", "frac": ach / PEAK_MFMA_BF16,
                 "traffic": MEASURED_TRAFFIC_BYTES.get(("train", lg)), "kernel": "mlp_train_fused_kernel (forward + loss + backward + partial dW)",
-                "kernel_ms": kern_ms, "algorithmic_flops_per_launch": flops}
+                "kernel_ms": kern_ms, "algorithmic_flops_per_launch": flops, "executed_flops_per_launch": executed,
+                "frac_executed": executed / (kern_ms * 1e-3) / 1e12 / PEAK_MFMA_BF16}
+        with_dx = {"what": "the same step with dL/dx requested: all 3 * n_mats products executed, dL/dx (M x 64 bf16) stored",
+                   "ms_per_step": step_dx_ms, "kernel_ms": kern_dx_ms, "frac": flops / (kern_dx_ms * 1e-3) / 1e12 / PEAK_MFMA_BF16,
+                   "mfma_frac_whole_step": flops / (step_dx_ms * 1e-3) / 1e12 / PEAK_MFMA_BF16}
         return line(METRIC, "samples/s", "bf16",
                     f"training step: w64, 4 hidden layers (5 matmuls), ReLU/linear, bf16, batch 2^{lg}, L2 loss, Adam on fp32 masters (BASELINE config 2)",
                     M, tm, self.K, self.Wm, self.args, roof,
-                    {"mfma_frac_whole_step": flops / (tm["ms"] * 1e-3) / 1e12 / PEAK_MFMA_BF16, "loss_first": loss0, "loss_last": float(loss.item())})
+                    {"mfma_frac_whole_step": flops / (tm["ms"] * 1e-3) / 1e12 / PEAK_MFMA_BF16,
+                     "mfma_frac_whole_step_executed": executed / (tm["ms"] * 1e-3) / 1e12 / PEAK_MFMA_BF16, "with_dLdx": with_dx,
+                     "loss_first": loss0, "loss_last": float(loss.item())})
 
-    def leg_infer(self, c):
+    def leg_infer(self, c, M=None, rotate=1, pf=None):
+        """M: rows of the timed call (the first M rows of the case's input). rotate: number of input / output buffer pairs the
+        calls cycle through; with enough of them (> 256 MB in all) no call finds its rows in the cache in front of the HBM.
+        pf: the prepared weights to run on (the initial ones for a leg whose output is compared with the checked one)."""
         np, torch, t, lib = self.np, self.torch, self.t, self.lib
         from tiny_dpcpp_nn.cabi import ptr
-        W, n_mats, M, desc = c["W"], c["n_mats"], c["M"], c["desc"]
-        y = torch.empty_like(c["x"])
+        W, n_mats, desc = c["W"], c["n_mats"], c["desc"]
+        M = M or c["M"]
+        pf = c["pf"] if pf is None else pf
+        xs = [c["x"][:M]] + [c["x"][:M].clone() for _ in range(rotate - 1)]
+        ys = [torch.empty_like(xs[0]) for _ in range(rotate)]
         s, d = t.stream(), ctypes.byref(desc)
-        a = (ptr(c["pf"]), ptr(c["x"]), ptr(y))
+        a = [(ptr(pf), ptr(x), ptr(y)) for x, y in zip(xs, ys)]
 
         def step(i):
-            if lib.tnn_mlp_inference(d, a[0], a[1], a[2], M, s):
+            b = a[i % rotate]
+            if lib.tnn_mlp_inference(d, b[0], b[1], b[2], M, s):
                 raise RuntimeError(lib.tnn_last_error())
 
         tm = self.timer().run(step)
+        same = None
+        if c.get("y_inference_checked") is not None and pf is not c["pf"]:
+            # rows are independent: this leg's output must be, bit for bit, the first M rows of the oracle-checked one
+            ref = torch.from_numpy(c["y_inference_checked"][:M]).to(t.dev).to(torch.bfloat16)
+            same = all(bool(torch.equal(y.view(torch.int16), ref.view(torch.int16))) for y in ys[: min(rotate, 2)])
+            if not same:
+                raise AssertionError("bench parity: this inference leg's rows differ from the checked full-batch output")
         flops = 2 * M * W * W * n_mats
         bytes_ = 2 * M * W * 2 + n_mats * W * W * 2
         lg = int(np.log2(M))
         ach = bytes_ / (tm["ms"] * 1e-3) / 1e9
         roof = {"bound": "hbm", "achieved": ach, "peak": PEAK_HBM, "unit": "GB/s", "frac": ach / PEAK_HBM,
-                "traffic": MEASURED_TRAFFIC_BYTES.get(("infer", lg)), "kernel": "mlp_forward_kernel (inference)", "kernel_ms": tm["ms"],
-                "algorithmic_bytes_per_launch": bytes_, "mfma_frac": flops / (tm["ms"] * 1e-3) / 1e12 / PEAK_MFMA_BF16}
+                "traffic": MEASURED_TRAFFIC_BYTES.get(("infer", lg)) if rotate == 1 else None, "kernel": "mlp_forward_kernel (inference)",
+                "kernel_ms": tm["ms"], "algorithmic_bytes_per_launch": bytes_, "mfma_frac": flops / (tm["ms"] * 1e-3) / 1e12 / PEAK_MFMA_BF16,
+                "buffers_in_rotation_bytes": rotate * 2 * M * W * 2}
+        extra = {"mfma_frac": roof["mfma_frac"]}
+        if same is not None:
+            extra["rows_bit_equal_to_checked_output"] = same
         return line(METRIC, "samples/s", "bf16",
-                    f"inference: w64, 4 hidden layers (5 matmuls), ReLU/linear, bf16, batch 2^{lg} (BASELINE config 1 shape)",
-                    M, tm, self.K, self.Wm, self.args, roof, {"mfma_frac": roof["mfma_frac"]})
+                    f"inference: w64, 4 hidden layers (5 matmuls), ReLU/linear, bf16, batch 2^{lg} (BASELINE config 1" +
+                    (")" if lg == 17 else " shape)") +
+                    (f"; {rotate} input/output buffer pairs in rotation, {rotate * 2 * M * W * 2 >> 20} MiB in all: no call finds its rows in the "
+                     "256 MB cache in front of the HBM" if rotate > 1 else "; one buffer pair (67 MB at 2^18 rows: it stays in that cache between calls)"),
+                    M, tm, self.K, self.Wm, self.args, roof, extra)
 
     # --------------------------------------------------------------------------------------------------------------
     def grid_case(self):
@@ -522,6 +578,11 @@ class Bench:
                 "kernel": ("grid_mlp_inference_kernel" if fused_mlp else "grid_forward_kernel") + (" over points in cell order" if ordered else ""),
                 "kernel_ms": kern_ms, "algorithmic_bytes_per_launch": bpp * M,
                 "frac_whole_step": bpp * M / (tm["ms"] * 1e-3) / 1e9 / PEAK_HBM}
+        # A 4-byte gather moves a whole 128-byte line: the bytes the memory side actually moved per launch (`traffic`, from the
+        # counters) over the kernel's time, as a fraction of the same peak. `frac` says how far the kernel is from the algorithmic
+        # ideal, this one how busy the memory system is.
+        if roof["traffic"]:
+            roof["frac_lines_moved"] = roof["traffic"] / (kern_ms * 1e-3) / 1e9 / PEAK_HBM
         out = line("hash-grid + fused-MLP inference points/s (3-D, 16x2, log2 22, fp16; w64, 3 hidden layers; batch 2^21); % HBM peak" if fused_mlp else
                    "hash-grid forward points/s (3-D, 16x2, log2 22, fp16 table, batch 2^21); % HBM peak", "points/s", "f16",
                    (f"3-D hash-grid encoding + w64/3-hidden-layer network inference in one kernel, 2^{lg} points (BASELINE config 5)" if fused_mlp else
@@ -788,10 +849,20 @@ def main():
         inf.update({"parity_checked": parity is not None, "parity": parity})
         if do_cpu:
             inf["cpu_baseline"] = cpu_baseline_infer(oracle, c["W"], c["n_mats"], budget_s=6.0 if wl == "all" else 12.0)
+        # config 1 at its own batch (2^17) and the 2^18 batch over six buffer pairs (402 MB), both on the initial weights so
+        # that their rows can be compared with the oracle-checked output
+        pf0 = b.t.prepare_packed(c["desc"], c["master0"], src_is_fp32=True)[0]
+        inf17 = b.leg_infer(c, M=1 << 17, pf=pf0)
+        inf_hbm = b.leg_infer(c, rotate=6, pf=pf0)
+        keep2 = ("value", "ms_per_step", "ms_per_step_reps", "config", "roofline", "mfma_frac", "rows_bit_equal_to_checked_output")
         if wl == "all":
             out["infer"] = sub(inf)
+            out["infer_2p17"] = {k: inf17[k] for k in keep2 if k in inf17}
+            out["infer_hbm"] = {k: inf_hbm[k] for k in keep2 if k in inf_hbm}
         else:
             out = inf
+            out["infer_2p17"] = {k: inf17[k] for k in keep2 if k in inf17}
+            out["infer_hbm"] = {k: inf_hbm[k] for k in keep2 if k in inf_hbm}
     if wl == "train_w128":
         out, W128, n_mats128 = b.leg_train_w128()
         out.update({"parity_checked": False, "parity": None})

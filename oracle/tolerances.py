@@ -46,6 +46,17 @@ def assert_close(a, b, dtype, what="", scale=1.0, frac_ok=0.0):
                              f"got {a[i]!r}, oracle {b[i]!r}")
 
 
+def bar_report(a, b, dtype, scale=1.0):
+    """How a result stands against the strict elementwise bar: the number of elements outside it, that number as a fraction,
+    and the worst ratio |a - b| / (atol * scale + rtol * |b|) (at most 1 when every element is inside)."""
+    a = np.asarray(a, np.float64)
+    b = np.asarray(b, np.float64)
+    atol, rtol = ELEMENTWISE[dtype]
+    ratio = np.abs(a - b) / (atol * scale + rtol * np.abs(b))
+    n_out = int((ratio > 1.0).sum())
+    return {"n": int(a.size), "n_outside": n_out, "frac_outside": n_out / max(int(a.size), 1), "worst_ratio": float(ratio.max()) if a.size else 0.0}
+
+
 def max_norm_rel(a, b):
     a = np.asarray(a, np.float64)
     b = np.asarray(b, np.float64)

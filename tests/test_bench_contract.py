@@ -50,6 +50,22 @@ def test_default_run_carries_the_whole_metric():
         check_roofline(out[leg]["roofline"])
         assert out[leg]["roofline"]["bound"] == "hbm"
     assert 0 < out["infer"]["roofline"]["mfma_frac"] < 1
+    # config 1 at its own batch, and the 2^18 batch over enough buffers that no call finds its rows in the cache
+    assert "2^17" in out["infer_2p17"]["config"]["workload"] and out["infer_2p17"]["config"]["batch"] == 1 << 17
+    assert out["infer_hbm"]["roofline"]["buffers_in_rotation_bytes"] > 256e6
+    for leg in ("infer_2p17", "infer_hbm"):
+        check_roofline(out[leg]["roofline"])
+        assert out[leg]["rows_bit_equal_to_checked_output"] is True
+    # the step executes 14 of the 15 products the convention counts (no dL/dx buffer); both fractions and a timing with dL/dx
+    roof = out["roofline"]
+    assert roof["executed_flops_per_launch"] * 15 == roof["algorithmic_flops_per_launch"] * 14
+    assert abs(roof["frac_executed"] * 15 - roof["frac"] * 14) < 1e-9
+    assert out["with_dLdx"]["kernel_ms"] > 0 and 0 < out["with_dLdx"]["frac"] < 1
+    # how many elements actually leave the strict elementwise bar
+    for what in ("y", "dW", "dLdx"):
+        rep = out["parity"]["strict_bar"][what]
+        assert rep["n"] > 0 and rep["frac_outside"] <= 2e-3 and rep["worst_ratio"] <= 4.0
+    assert "frac_lines_moved" in out["grid"]["roofline"]
 
 
 @pytest.mark.gpu

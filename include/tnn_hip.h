@@ -214,6 +214,22 @@ int tnn_mlp_train_step_l2_adam(const tnn_mlp_desc *desc, void *d_prepared_fwd, v
                                void *d_dLdx, size_t M, void *d_workspace, size_t workspace_bytes, void *main_kernel_done_event,
                                tnn_stream_t stream);
 
+/* Network::backward_pass (include/network/SwiftNetMLP.h:199-257 over kernel_esimd.h:160-240) for a caller that kept no
+ * activations: the weight gradients (and dL/dx) for a given dL/dy, with the forward pass formed again on chip from d_x in the
+ * same kernel. It pairs with tnn_mlp_inference as the forward pass of a training step whose loss is computed by the caller
+ * (PyTorch autograd): no M x W matrix except x, y and dL/dy is written or read, where forward_pass + backward_pass move
+ * 2 * (n_hidden_layers + 2) of them. Same values as tnn_mlp_forward + tnn_mlp_backward on the same inputs (the activations
+ * are the same bits; the weight gradients are fp32 sums over the batch taken in this kernel's fixed order).
+ *   d_dLdy: M x W of T, the derivative of the loss with respect to the ACTIVATED output (the output activation's derivative
+ *   is applied here, as in backward_pass). d_dW: raw layout [out][in], fp32 or T. d_dLdx: NULL or M x W of T.
+ * Shapes: those of the one-kernel training step (width 16 / 32 / 64, up to 5 matrices at width 64 and 6 below);
+ * tnn_mlp_backward_recompute_supported returns TNN_OK for them and TNN_ERR_UNSUPPORTED otherwise, and such a network
+ * keeps its activations (tnn_mlp_forward + tnn_mlp_backward). Workspace: tnn_mlp_train_step_workspace_bytes. */
+int tnn_mlp_backward_recompute_supported(const tnn_mlp_desc *desc);
+int tnn_mlp_backward_recompute(const tnn_mlp_desc *desc, const void *d_prepared_fwd, const void *d_prepared_bwd, const void *d_x,
+                               const void *d_dLdy, void *d_dW, int dW_is_fp32, void *d_dLdx, size_t M, void *d_workspace,
+                               size_t workspace_bytes, tnn_stream_t stream);
+
 /* Testing aid, no counterpart in the reference. In the width-64 training and backward kernels the four waves that share
  * staged tiles meet at a counter in LDS; a wave waits there for at most `iterations` polls (default 2^22, far beyond any
  * real wait) so that a kernel always ends. A wave whose wait runs out marks its workgroup, and the call then delivers NaN
@@ -373,6 +389,16 @@ int tnn_grid_mlp_train_step_l2_adam(const tnn_grid_desc *grid, const tnn_mlp_des
                                     float loss_scale, void *d_y, float *d_loss_sum, float *d_master_packed, float *d_m, float *d_v,
                                     int step, float lr, float beta1, float beta2, float eps, void *d_packed_T, float *d_grad_table,
                                     int overwrite, size_t M, void *d_workspace, size_t workspace_bytes, tnn_stream_t stream);
+/* The backward pass of a network behind a hash-grid encoding for a given dL/dy, without the encoded matrix: what
+ * loss.backward() does through NetworkWithInputEncoding in the reference (dpcpp_bindings/tiny_dpcpp_nn/modules.py:84-136 over
+ * Network::backward_pass and GridEncoding::backward_impl, include/encodings/grid.h:752-797). The encoding and the
+ * network's forward pass are formed again on chip from the positions (tnn_grid_mlp_inference is the forward pass that goes
+ * with it), the weight gradients leave as in tnn_mlp_backward_recompute, and dL/d(encoding) goes through the workspace into
+ * the scatter of tnn_grid_backward (tnn_grid_backward_ordered when d_order is given). d_grad_table: n_params fp32, or NULL
+ * when only the network's gradients are wanted. Shapes and workspace as tnn_grid_mlp_train_step_l2_adam. */
+int tnn_grid_mlp_backward(const tnn_grid_desc *grid, const tnn_mlp_desc *mlp, const float *d_x, const void *d_order, const void *d_table,
+                          const void *d_prepared_fwd, const void *d_prepared_bwd, const void *d_dLdy, void *d_dW, int dW_is_fp32,
+                          float *d_grad_table, int overwrite, size_t M, void *d_workspace, size_t workspace_bytes, tnn_stream_t stream);
 /* TNN_OK when tnn_grid_mlp_inference runs this pair of shapes, otherwise the status (and tnn_last_error the reason) it
  * would return: lets a caller choose between the fused call and the two calls once, when the modules are built. */
 int tnn_grid_mlp_supported(const tnn_grid_desc *grid, const tnn_mlp_desc *mlp);

@@ -4,7 +4,7 @@ import ctypes
 import numpy as np
 import pytest
 
-from tolerances import BF16, FP16, assert_close, assert_propagated, max_norm_rel
+from tolerances import BF16, FP16, PROPAGATED, assert_close, assert_propagated, max_norm_rel
 
 pytestmark = pytest.mark.gpu
 
@@ -511,3 +511,52 @@ def test_train_step_is_reproducible(tnn, oracle, dtype, W, n_hidden, log2_m):
         else:
             for a, b in zip(got, first):
                 assert torch.equal(a.view(torch.int16 if a.element_size() == 2 else torch.int32), b.view(torch.int16 if b.element_size() == 2 else torch.int32))
+
+
+@pytest.mark.parametrize("dtype,W,n_hidden,act,out_act,M", [
+    (BF16, 64, 4, "relu", "none", 1 << 14), (BF16, 64, 4, "relu", "none", 8), (FP16, 64, 2, "relu", "relu", 4104),
+    (FP16, 64, 1, "sigmoid", "sigmoid", 1000 * 8), (BF16, 32, 4, "relu", "none", 3 * 4096 + 8), (FP16, 32, 5, "none", "none", 2048),
+    (FP16, 16, 2, "relu", "sigmoid", 777 * 8), (BF16, 16, 5, "sigmoid", "none", 4096)])
+def test_backward_recompute_equals_forward_plus_backward(tnn, oracle, dtype, W, n_hidden, act, out_act, M):
+    """The backward pass that forms the activations again on chip (tnn_mlp_backward_recompute, the backward half of a training
+    step whose loss the caller computes) against forward_pass + backward_pass on the same inputs: dL/dx bit for bit (the same
+    rounded chain per row), the weight gradients to the rounding of fp32 sums taken in another order, and both against the
+    oracle (Network::backward_pass, include/network/kernel_esimd.h:160-240)."""
+    import torch
+    n_mats = n_hidden + 1
+    w, x = make_case(oracle, dtype, W, n_mats, M)
+    rng = np.random.default_rng(M + W)
+    g = oracle.round(rng.standard_normal((M, W)) * 0.05, dtype)
+    desc = tnn.mlp_desc(dtype, W, n_hidden, act, out_act)
+    assert tnn.lib.tnn_mlp_backward_recompute_supported(ctypes.byref(desc)) == 0
+    _, pf, pb = tnn.prepare(desc, w)
+    xt, gt = tnn.dev_tensor(x, dtype), tnn.dev_tensor(g, dtype)
+    interm = tnn.forward(desc, pf, xt)
+    _, dW_ref, dX_ref = tnn.backward(desc, pb, gt, interm, dw_fp32=True)
+    dW, dX = tnn.backward_recompute(desc, pf, pb, xt, gt)
+    assert torch.equal(dX.view(torch.int16), dX_ref.view(torch.int16)), "dL/dx differs from forward_pass + backward_pass"
+    scale = float(dW_ref.abs().max())
+    assert torch.allclose(dW, dW_ref, rtol=1e-4, atol=1e-5 * scale), float((dW - dW_ref).abs().max())
+    ri = oracle.mlp_forward_T(dtype, W, n_mats, act, out_act, w, x)
+    _, rdW, rdX = oracle.mlp_backward_T(dtype, W, n_mats, act, out_act, w, ri, g, round_dw=False)
+    assert_propagated(tnn.host(dW), rdW, dtype, "dW of the recompute backward", scale=float(np.abs(rdW).max()))
+    assert_close(tnn.host(dX), rdX, dtype, "dL/dx of the recompute backward", scale=float(np.abs(rdX).max()), frac_ok=PROPAGATED)
+    # without dL/dx, and with the gradients in the network's type
+    dW2, none = tnn.backward_recompute(desc, pf, pb, xt, gt, want_dx=False, dw_fp32=False)
+    assert none is None and torch.equal(dW2.view(torch.int16), dW.to(dW2.dtype).view(torch.int16))
+
+
+def test_backward_recompute_rejects_what_it_cannot_run(tnn):
+    from tiny_dpcpp_nn import _lib
+    wide = tnn.mlp_desc(FP16, 128, 2, "relu", "none")
+    deep = tnn.mlp_desc(BF16, 64, 7, "relu", "none")
+    for d in (wide, deep):
+        assert tnn.lib.tnn_mlp_backward_recompute_supported(ctypes.byref(d)) == _lib.TNN_ERR_UNSUPPORTED
+    ok = tnn.mlp_desc(BF16, 64, 2, "relu", "none")
+    import torch
+    t = torch.zeros((8, 64), dtype=torch.bfloat16, device=tnn.dev)
+    ws = torch.empty(16, dtype=torch.uint8, device=tnn.dev)
+    from gpu_harness import ptr
+    assert tnn.lib.tnn_mlp_backward_recompute(ctypes.byref(ok), ptr(t), ptr(t), ptr(t), ptr(t), ptr(t), 1, None, 8, ptr(ws), 16, tnn.stream()) == _lib.TNN_ERR_WORKSPACE
+    assert tnn.lib.tnn_mlp_backward_recompute(ctypes.byref(ok), ptr(t), ptr(t), ptr(t), None, ptr(t), 1, None, 8, ptr(ws), 16, tnn.stream()) == _lib.TNN_ERR_INVALID_ARGUMENT
+    assert tnn.lib.tnn_mlp_backward_recompute(ctypes.byref(ok), ptr(t), ptr(t), ptr(t), ptr(t), ptr(t), 1, None, 12, ptr(ws), 16, tnn.stream()) == _lib.TNN_ERR_INVALID_ARGUMENT

@@ -323,6 +323,106 @@ def test_network_with_input_encoding_trains(tcnn, dtype):
         model.get_params()
 
 
+@pytest.mark.parametrize("dtype,width,n_hidden,act,out_act,batch", [
+    (torch.bfloat16, 64, 4, "relu", "none", 4096), (torch.float16, 64, 2, "relu", "sigmoid", 1000), (torch.float16, 32, 3, "sigmoid", "none", 520),
+    (torch.bfloat16, 16, 5, "relu", "relu", 8)])
+def test_training_without_stored_activations_equals_the_stored_route(tcnn, dtype, width, n_hidden, act, out_act, batch):
+    """A network whose shape has the one-kernel backward pass trains without stored activations: inference() forward,
+    bwd_recompute() backward. Against the reference's route on the same native module (fwd() keeps every activation,
+    bwd_no_encoding_grad() reads them): the output and dL/dx bit for bit, the weight gradients -- sums over the batch, rounded
+    to the network's type, taken in another order -- to a unit in the last place."""
+    torch.manual_seed(batch)
+    net = tcnn.Network(width, width, net_config(width, n_hidden, act, out_act), dtype=dtype, use_bias=False)
+    native = net.tnn_module
+    assert native.can_recompute_backward()
+    x = (torch.rand((batch, width), device=DEVICE) * 2 - 1).to(dtype)
+    dy = ((torch.rand((batch, width), device=DEVICE) * 2 - 1) * 0.1).to(dtype)
+    y_stored = native.fwd(x)
+    dx_stored, dw_stored = native.bwd_no_encoding_grad(dy, True, True)
+    y = native.inference(x)
+    dx, dw = native.bwd_recompute(dy, x, True, True)
+    assert torch.equal(y.view(torch.int16), y_stored.view(torch.int16))
+    assert torch.equal(dx.view(torch.int16), dx_stored.view(torch.int16))
+    scale = float(dw_stored.float().abs().max())
+    assert torch.allclose(dw.float(), dw_stored.float(), rtol=2 ** -7 if dtype == torch.bfloat16 else 2 ** -10, atol=1e-4 * scale)
+    assert float((dw.view(torch.int16) != dw_stored.view(torch.int16)).float().mean()) < 0.02
+    _, dw_only = native.bwd_recompute(dy, x, True, False)
+    assert torch.equal(dw_only.view(torch.int16), dw.view(torch.int16))
+    # the module takes that route by itself, in training and in evaluation mode, and two forward passes may precede their
+    # backward passes (nothing of a forward pass is kept in the module)
+    net.train()
+    xa, xb = x[: batch // 2 + 4].float().requires_grad_(True), x.float().requires_grad_(True)
+    ya, yb = net(xa), net(xb)
+    (ya.float().square().mean() + yb.float().square().mean()).backward()
+    assert xa.grad is not None and xb.grad is not None and net.params.grad is not None and torch.isfinite(net.params.grad).all()
+    wide = tcnn.Network(128, 128, net_config(128, 2), dtype=torch.float16)
+    assert not wide.tnn_module.can_recompute_backward()
+    with pytest.raises(Exception, match="not available|no fused training kernel"):
+        wide.tnn_module.bwd_recompute(torch.zeros((8, 128), dtype=torch.float16, device=DEVICE), torch.zeros((8, 128), dtype=torch.float16, device=DEVICE), True, False)
+
+
+@pytest.mark.parametrize("dtype,n_dims,grid,n_hidden,batch", [
+    (torch.float16, 2, GRID_2D, 2, 4096), (torch.bfloat16, 2, GRID_2D, 1, 1001),
+    (torch.float16, 3, {"otype": "HashGrid", "n_levels": 16, "n_features_per_level": 2, "log2_hashmap_size": 14, "base_resolution": 16, "per_level_scale": 1.447}, 3, 2048)])
+def test_network_with_grid_encoding_trains_through_one_kernel(tcnn, oracle, dtype, n_dims, grid, n_hidden, batch):
+    """NetworkWithInputEncoding with autograd on a grid encoding: forward is the fused inference kernel, backward one kernel
+    that forms encoding and activations again plus the scatter. Against the two modules in turn (the reference's only route,
+    dpcpp_bindings/tiny_dpcpp_nn/modules.py:389-407) on the same model: output bit for bit, network gradients to a unit in the
+    last place of the network's type, table gradients to 1e-5 of their largest; and against the oracle's chain."""
+    torch.manual_seed(17)
+    model = tcnn.NetworkWithInputEncoding(n_dims, 3, net_config(64, n_hidden), dict(grid), dtype=dtype, use_bias=False)
+    with torch.no_grad():
+        model.encoding.params.copy_(torch.rand_like(model.encoding.params) * 2 - 1)
+    model.train()
+    assert model.network.tnn_module.can_train_with_encoding(model.encoding.tnn_module)
+    x = torch.rand((batch, n_dims), device=DEVICE)
+    target = torch.rand((batch, 3), device=DEVICE)
+
+    def grads(run):
+        model.zero_grad(set_to_none=True)
+        out = run(x)
+        ((out.float() - target) ** 2).mean().backward()
+        return out.detach(), model.network.params.grad.clone(), model.encoding.params.grad.clone()
+
+    y2, dnet2, dtab2 = grads(model.network_with_encoding)   # Encoding.forward, then Network.forward
+    y1, dnet1, dtab1 = grads(model)                        # one kernel each way
+    assert y1.shape == (batch, 3) and y1.dtype == dtype
+    assert torch.equal(y1.view(torch.int16), y2.view(torch.int16))
+    net_scale, tab_scale = float(dnet2.abs().max()), float(dtab2.abs().max())
+    assert net_scale > 0 and tab_scale > 0
+    assert torch.allclose(dnet1, dnet2, rtol=2 ** -7 if dtype == torch.bfloat16 else 2 ** -10, atol=1e-4 * net_scale), float((dnet1 - dnet2).abs().max()) / net_scale
+    # bf16 (loss scale 1): the same dL/d(encoding) bits go into the scatter on both routes, only the order of the atomic
+    # additions differs. fp16 (loss scale 128): the two-module route divides dL/d(encoding) by the loss scale in fp16 before
+    # the scatter, which pushes it into the subnormal range and costs it bits (about 1e-3 of the largest gradient here);
+    # the fused route scatters the scaled values and divides the fp32 sums, which is the more accurate of the two -- the
+    # oracle's chain below is the judge of both.
+    assert float((dtab1 - dtab2).abs().max()) <= (2e-3 if dtype == torch.float16 else 1e-5) * tab_scale, float((dtab1 - dtab2).abs().max()) / tab_scale
+    # the oracle's chain: encoding (fp32 table) rounded to the network's type, network forward, backward with dL/d(encoding), scatter
+    W, n_mats = 64, n_hidden + 1
+    T = DT[dtype]
+    cfg = oracle_cfg(grid, n_dims)
+    table = model.encoding.params.detach().cpu().numpy().reshape(-1)
+    w = oracle.round(unpack(model.network.get_params().float().cpu().numpy().reshape(-1), n_mats, W), T)
+    enc = oracle.round(oracle.grid_forward(cfg, table, x.cpu().numpy(), W), T)
+    interm = oracle.mlp_forward_T(T, W, n_mats, "relu", "none", w, enc)
+    assert_propagated(y1.float().cpu().numpy(), interm[-1][:, :3], T, "fused output against the oracle chain")
+    scale = model.network.loss_scale
+    dy = np.zeros((batch, W), np.float32)
+    dy[:, :3] = (2.0 / (3 * batch)) * (y1.float().cpu().numpy() - target.cpu().numpy()) * scale
+    dy = oracle.round(dy, T)
+    _, rdW, rd_enc = oracle.mlp_backward_T(T, W, n_mats, "relu", "none", w, interm, dy, round_dw=False)
+    ref_tab = oracle.grid_backward(cfg, x.cpu().numpy(), rd_enc, table.size) / scale
+    assert max_norm_rel(dtab1.cpu().numpy().reshape(-1), ref_tab) <= (1e-2 if dtype == torch.bfloat16 else 5e-3)
+    # rdW is raw [out][in]; the module's gradient is packed [in][out]
+    got = unpack(dnet1.float().cpu().numpy().reshape(-1), n_mats, W)
+    assert max(max_norm_rel(got[l], rdW[l].T / scale) for l in range(n_mats)) <= (1e-2 if dtype == torch.bfloat16 else 5e-3)
+    # evaluation mode with autograd takes the same route; positions get no gradient
+    model.eval()
+    xg = x.clone().requires_grad_(True)
+    model(xg).float().sum().backward()
+    assert xg.grad is None
+
+
 def test_parameter_free_encodings_through_the_package(tcnn, oracle):
     """test/python/test_encodings.py:377-630 of the reference: spherical harmonics (golden rows), identity, padding, frequency."""
     import json
@@ -415,7 +515,7 @@ def test_training_through_data_writes(tcnn):
         opt.zero_grad()
         loss.backward()
         opt.step()
-        losses.append(float(loss))
+        losses.append(float(loss.detach()))
         outputs.append(y.detach().clone())
     assert not torch.equal(outputs[0], outputs[1]), "a step written through .data did not reach the kernels"
     assert losses[-1] < 0.05 * losses[0], losses

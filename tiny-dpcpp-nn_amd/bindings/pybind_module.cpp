@@ -59,6 +59,20 @@ class PybindingModule {
         CHECK_INPUT(positions);
         return m_module->inference_with_encoding(*encoding.m_module, positions);
     }
+    /// Network modules, training without stored activations: inference() is the forward pass, these are the backward passes.
+    bool can_recompute_backward() const { return m_module->can_recompute_backward(); }
+    std::tuple<torch::Tensor, torch::Tensor> bwd_recompute(torch::Tensor grad_output, torch::Tensor input_from_fwd, bool pack_gradient, bool get_dl_dinput) {
+        CHECK_INPUT(grad_output);
+        CHECK_INPUT(input_from_fwd);
+        return m_module->backward_pass_recompute(grad_output, input_from_fwd, pack_gradient, get_dl_dinput);
+    }
+    bool can_train_with_encoding(const PybindingModule &encoding) const { return m_module->can_train_with_encoding(*encoding.m_module); }
+    std::tuple<torch::Tensor, torch::Tensor> bwd_with_encoding(const PybindingModule &encoding, torch::Tensor positions, torch::Tensor grad_output,
+                                                               bool pack_gradient) {
+        CHECK_INPUT(positions);
+        CHECK_INPUT(grad_output);
+        return m_module->backward_with_encoding(*encoding.m_module, positions, grad_output, pack_gradient);
+    }
     torch::Tensor initial_params() { return m_module->initialize_params(); }
     torch::Tensor initial_params(torch::Tensor &tensor) { return m_module->initialize_params(tensor); }
     /// weights_are_packed: the tensor already is in the packed parameter layout, no packing is done
@@ -116,6 +130,10 @@ PYBIND11_MODULE(tiny_dpcpp_nn_pybind_module, m) {
         .def("inference", &PybindingModule::inference)
         .def("can_fuse_encoding", &PybindingModule::can_fuse_encoding)
         .def("inference_with_encoding", &PybindingModule::inference_with_encoding)
+        .def("can_recompute_backward", &PybindingModule::can_recompute_backward)
+        .def("bwd_recompute", &PybindingModule::bwd_recompute)
+        .def("can_train_with_encoding", &PybindingModule::can_train_with_encoding)
+        .def("bwd_with_encoding", &PybindingModule::bwd_with_encoding)
         .def("bwd_no_encoding_grad", &PybindingModule::bwd_no_encoding_grad)
         .def("bwd_with_encoding_grad", &PybindingModule::bwd_with_encoding_grad)
         .def("initial_params", py::overload_cast<>(&PybindingModule::initial_params))

@@ -64,6 +64,8 @@ struct TrainTail {
     bool use_adam = false;       // apply Adam to the reduced gradients inside the reduction kernel
     AdamArgs adam{};
     hipEvent_t main_done = nullptr; // recorded between the main kernel and the reduction when not null
+    void *dW = nullptr;             // launchers that have no dW argument of their own: where the reduced gradients go, if anywhere
+    int dW_is_fp32 = 1;
 };
 
 } // namespace tnn

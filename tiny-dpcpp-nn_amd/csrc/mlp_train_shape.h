@@ -45,6 +45,12 @@ int fused_train_launch_fp16(const tnn_mlp_desc *d, const FusedPlan &p, const voi
                             const float *targets, float loss_scale, void *y, float *loss_sum, void *dW, int dW_is_fp32, void *dx,
                             size_t M, float *partials, float *loss_partials, const TrainTail &tail, hipStream_t s);
 
+// The same kernels with dL/dy given by the caller (mlp_train_given_*.hip): backward pass with the activations formed again on chip.
+int fused_given_launch_bf16(const tnn_mlp_desc *d, const FusedPlan &p, const void *wf, const void *wb, const void *x, const void *dLdy, void *dW,
+                            int dW_is_fp32, void *dx, size_t M, float *partials, float *loss_partials, hipStream_t s);
+int fused_given_launch_fp16(const tnn_mlp_desc *d, const FusedPlan &p, const void *wf, const void *wb, const void *x, const void *dLdy, void *dW,
+                            int dW_is_fp32, void *dx, size_t M, float *partials, float *loss_partials, hipStream_t s);
+
 // Backward pass with the weight gradients in the same kernel (mlp_backward_fused.inc). TNN_ERR_UNSUPPORTED when the shape has
 // no such kernel or the workspace holds no partial tile; the caller then runs the separate kernels.
 int fused_backward(const tnn_mlp_desc *d, const void *wb, const void *dLdy, const void *interm_fwd, void *interm_bwd, void *dW,

@@ -1,7 +1,6 @@
 // One training step of the fused MLP against an L2 loss: forward, loss + gradient, backward with
 // weight gradients (include/trainer.h:23-46 with include/losses/l2.h:19-40 in between).
-#include "adam_update.h"
-#include "tnn_internal.h"
+#include "mlp_train_shape.h"
 
 #include <mutex>
 
@@ -140,6 +139,32 @@ TNN_API int tnn_mlp_train_step_l2_adam(const tnn_mlp_desc *desc, void *d_prepare
     if (tail.main_done && hipEventRecord(tail.main_done, s) != hipSuccess) return fail(TNN_ERR_HIP, "hipEventRecord failed");
     return tnn_mlp_adam_update(desc, d_master_packed, d_m, d_v, dW, 1.0f / loss_scale, step, lr, beta1, beta2, eps, d_packed_T,
                                d_prepared_fwd, d_prepared_bwd, stream);
+}
+
+TNN_API int tnn_mlp_backward_recompute_supported(const tnn_mlp_desc *desc) {
+    int rc = check_mlp_desc(desc);
+    if (rc) return rc;
+    if (!fused_plan(desc, 8).supported) return fail(TNN_ERR_UNSUPPORTED, "no fused training kernel for width %d with %d matrices", desc->width, desc->n_hidden_layers + 1);
+    return TNN_OK;
+}
+
+TNN_API int tnn_mlp_backward_recompute(const tnn_mlp_desc *desc, const void *d_prepared_fwd, const void *d_prepared_bwd, const void *d_x,
+                                       const void *d_dLdy, void *d_dW, int dW_is_fp32, void *d_dLdx, size_t M, void *d_workspace,
+                                       size_t workspace_bytes, tnn_stream_t stream) {
+    int rc = tnn_mlp_backward_recompute_supported(desc);
+    if (rc) return rc;
+    if (!d_prepared_fwd || !d_prepared_bwd || !d_x || !d_dLdy || !d_dW) return fail(TNN_ERR_INVALID_ARGUMENT, "NULL pointer argument");
+    if (M == 0 || (M % 8) != 0) return fail(TNN_ERR_INVALID_ARGUMENT, "batch size %zu is not a positive multiple of 8", M);
+    const FusedPlan p = fused_plan(desc, M);
+    const size_t need = p.partial_bytes + p.loss_bytes + 512;
+    if (!d_workspace || workspace_bytes < need) return fail(TNN_ERR_WORKSPACE, "workspace of %zu bytes given, %zu needed", workspace_bytes, need);
+    const uintptr_t base = align256(reinterpret_cast<uintptr_t>(d_workspace));
+    float *loss_partials = reinterpret_cast<float *>(base);
+    float *partials = reinterpret_cast<float *>(base + p.loss_bytes);
+    hipStream_t s = as_stream(stream);
+    if (desc->dtype == TNN_BF16)
+        return fused_given_launch_bf16(desc, p, d_prepared_fwd, d_prepared_bwd, d_x, d_dLdy, d_dW, dW_is_fp32, d_dLdx, M, partials, loss_partials, s);
+    return fused_given_launch_fp16(desc, p, d_prepared_fwd, d_prepared_bwd, d_x, d_dLdy, d_dW, dW_is_fp32, d_dLdx, M, partials, loss_partials, s);
 }
 
 // ------------------------------------------------------------------------------------------------

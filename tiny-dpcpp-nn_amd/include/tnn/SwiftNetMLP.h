@@ -98,19 +98,65 @@ template <typename T, int WIDTH> class SwiftNetMLP : public Network<T> {
         RequireDense(input);
         if (dL_dinput != nullptr) RequireDense(*dL_dinput);
         const tnn_mlp_desc d = desc();
-        const size_t need = tnn_mlp_backward_workspace_bytes(&d, input.m());
-        if (need > workspace_bytes_) {
-            this->get_queue().wait();
-            tnn::detail::device_free(workspace_);
-            workspace_ = nullptr;
-            workspace_bytes_ = 0;
-            tnn::hip_check(hipMalloc(&workspace_, need), "hipMalloc");
-            workspace_bytes_ = need;
-        }
+        ReserveWorkspace(tnn_mlp_backward_workspace_bytes(&d, input.m()));
         tnn::abi_check(tnn_mlp_backward(&d, this->prepared_backward(), input.GetPointer(), intermediate_output_forward.GetMatrixPointer(0),
                                         intermediate_output_backward.GetMatrixPointer(0), output.GetMatrixPointer(0), 0,
                                         dL_dinput ? dL_dinput->GetPointer() : nullptr, input.m(), workspace_, workspace_bytes_,
                                         this->get_queue().abi()));
+        return {tnn::event(this->get_queue().get())};
+    }
+
+    /// Whether backward_pass_recompute runs for this network (the shapes of the one-kernel training step).
+    bool supports_backward_recompute() const {
+        const tnn_mlp_desc d = desc();
+        return Network<T>::get_input_width() == WIDTH && tnn_mlp_backward_recompute_supported(&d) == TNN_OK;
+    }
+
+    /// backward_pass for a caller that kept no activations: weight gradients (raw layout, as backward_pass writes them) and,
+    /// on request, dL/dinput for `dL_doutput`, the activations being formed again on chip from `input` (the matrix the
+    /// forward pass ran on; inference() is the forward pass that goes with this). No counterpart in the reference, whose
+    /// backward_pass reads interm_forw (include/network/SwiftNetMLP.h:199-257); same values.
+    std::vector<tnn::event> backward_pass_recompute(const DeviceMatrixView<T> input, const DeviceMatrixView<T> dL_doutput, DeviceMatricesView<T> output,
+                                                    DeviceMatrixView<T> *dL_dinput = nullptr) {
+        RequireDense(input);
+        RequireDense(dL_doutput);
+        if (dL_dinput != nullptr) RequireDense(*dL_dinput);
+        if (input.m() != dL_doutput.m()) throw std::invalid_argument("input and dL_doutput differ in their number of rows.");
+        const tnn_mlp_desc d = desc();
+        ReserveWorkspace(tnn_mlp_train_step_workspace_bytes(&d, input.m()));
+        tnn::abi_check(tnn_mlp_backward_recompute(&d, this->prepared_forward(), this->prepared_backward(), input.GetPointer(), dL_doutput.GetPointer(),
+                                                  output.GetMatrixPointer(0), 0, dL_dinput ? dL_dinput->GetPointer() : nullptr, input.m(), workspace_,
+                                                  workspace_bytes_, this->get_queue().abi()));
+        return {tnn::event(this->get_queue().get())};
+    }
+
+    /// Whether backward_with_grid runs for this grid.
+    bool supports_grid_training(const tnn_grid_desc &grid) const {
+        const tnn_mlp_desc d = desc();
+        return Network<T>::get_input_width() == WIDTH && tnn_grid_mlp_train_supported(&grid, &d) == TNN_OK;
+    }
+
+    /// The backward pass of this network behind a grid encoding of `positions`, for `dL_doutput`: weight gradients into `output`
+    /// (raw layout) and the table's gradient (fp32, overwritten) into `grad_table` when it is not null. Encoding and forward
+    /// pass are formed again on chip; the encoded matrix is never stored (inference_with_grid is the forward pass that goes
+    /// with this). Batches from 2^17 rows on are visited in cell order, as GridEncoding's own backward pass does.
+    std::vector<tnn::event> backward_with_grid(const tnn_grid_desc &grid, const void *table, const float *positions, const DeviceMatrixView<T> dL_doutput,
+                                               DeviceMatricesView<T> output, float *grad_table) {
+        RequireDense(dL_doutput);
+        const size_t M = dL_doutput.m();
+        const tnn_mlp_desc d = desc();
+        ReserveWorkspace(tnn_grid_mlp_train_step_workspace_bytes(&grid, &d, M));
+        const void *order = nullptr;
+        if (M >= (size_t(1) << 17)) {
+            const size_t bytes = tnn_grid_order_bytes(&grid, M);
+            if (!m_grid_order || m_grid_order->size() * sizeof(float) < bytes)
+                m_grid_order = std::make_unique<DeviceMatrix<float>>((bytes + sizeof(float) - 1) / sizeof(float), 1, this->get_queue());
+            tnn::abi_check(tnn_grid_order_points(&grid, positions, M, m_grid_order->data(), m_grid_order->size() * sizeof(float), this->get_queue().abi()));
+            order = m_grid_order->data();
+        }
+        tnn::abi_check(tnn_grid_mlp_backward(&grid, &d, order ? nullptr : positions, order, table, this->prepared_forward(), this->prepared_backward(),
+                                             dL_doutput.GetPointer(), output.GetMatrixPointer(0), 0, grad_table, 1, M, workspace_, workspace_bytes_,
+                                             this->get_queue().abi()));
         return {tnn::event(this->get_queue().get())};
     }
 
@@ -123,6 +169,17 @@ template <typename T, int WIDTH> class SwiftNetMLP : public Network<T> {
         d.activation = tnn::to_abi(m_activation);
         d.output_activation = tnn::to_abi(m_output_activation);
         return d;
+    }
+
+    /// The workspace grows to the largest request seen; growing waits for the work that may still use the old one.
+    void ReserveWorkspace(const size_t need) {
+        if (need <= workspace_bytes_) return;
+        this->get_queue().wait();
+        tnn::detail::device_free(workspace_);
+        workspace_ = nullptr;
+        workspace_bytes_ = 0;
+        tnn::hip_check(hipMalloc(&workspace_, need), "hipMalloc");
+        workspace_bytes_ = need;
     }
 
     static void RequireDense(const DeviceMatrixView<T> &v) {

@@ -45,7 +45,7 @@ inline std::vector<float> numbers_of(const std::string &text, const std::string 
         if (after == p || (after < end && !separates_numbers(*after)))
             throw std::invalid_argument(origin + ": not a number at byte " + std::to_string(p - begin));
         // too large for a float, whether or not it fits a double (a text "inf" passes: it says what it means)
-        const bool spelled_inf = std::string(p, after).find_first_of("nN") != std::string::npos;
+        const bool spelled_inf = std::string(p, static_cast<size_t>(after - p)).find_first_of("nN") != std::string::npos;
         if (!spelled_inf && (v > std::numeric_limits<float>::max() || v < -std::numeric_limits<float>::max()))
             throw std::out_of_range(origin + ": number out of range at byte " + std::to_string(p - begin));
         out.push_back(static_cast<float>(v));

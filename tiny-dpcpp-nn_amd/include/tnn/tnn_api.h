@@ -60,6 +60,21 @@ class Module {
         throw std::runtime_error("inference_with_encoding: not a network module");
     }
 
+    /// Network modules, training without stored activations (no counterpart in the reference, whose forward_pass keeps
+    /// interm_forw for backward_pass, include/tnn_api.h:541-603): when can_recompute_backward() holds, a training step may run
+    /// inference() as its forward pass and backward_pass_recompute(grad_output, the same input, ...) as its backward pass; the
+    /// activations are formed again on chip. Same return value as backward_pass.
+    virtual bool can_recompute_backward() const { return false; }
+    virtual std::tuple<torch::Tensor, torch::Tensor> backward_pass_recompute(const torch::Tensor &, const torch::Tensor &, bool, bool) {
+        throw std::runtime_error("backward_pass_recompute: not available for this module");
+    }
+    /// The same behind a grid encoding: inference_with_encoding() is the forward pass, backward_with_encoding returns the
+    /// network's weight gradients (packed on request) and the gradient of the encoding's table.
+    virtual bool can_train_with_encoding(const Module &) const { return false; }
+    virtual std::tuple<torch::Tensor, torch::Tensor> backward_with_encoding(const Module &, const torch::Tensor &, const torch::Tensor &, bool) {
+        throw std::runtime_error("backward_with_encoding: not a network module");
+    }
+
     tnn::queue &get_queue() { return queue_; }
 
     /// First thing in every method: the module's kernels go to the stream the caller's tensor operations are on, so inputs
@@ -382,6 +397,50 @@ template <typename T, int WIDTH> class NetworkModule : public Module {
         return {input_grad, fromDevice<T>(result->GetViews().GetMatrixPointer(0), {(int64_t)result->nelements(), 1})};
     }
 
+    bool can_recompute_backward() const override { return network_.supports_backward_recompute(); }
+
+    std::tuple<torch::Tensor, torch::Tensor> backward_pass_recompute(const torch::Tensor &grad_output, const torch::Tensor &input_tensor,
+                                                                     bool pack_transpose_gradient, bool get_dl_dinput) override {
+        this->enter();
+        const size_t batch_size = CheckedBatch(input_tensor, network_.get_input_width());
+        CheckedGradOutput(grad_output, batch_size);
+        if (batch_size == 0) throw std::invalid_argument("backward_pass_recompute: empty batch");
+        DeviceMatrixView<T> input_dm(batch_size, network_.get_input_width(), network_.get_input_width(), reinterpret_cast<T *>(input_tensor.data_ptr()));
+        DeviceMatrixView<T> dL_doutput(batch_size, network_.get_output_width(), network_.get_output_width(), reinterpret_cast<T *>(grad_output.data_ptr()));
+        torch::Tensor input_grad;
+        if (get_dl_dinput)
+            input_grad = torch::empty({(int64_t)(batch_size * network_.get_input_width()), 1}, torch::TensorOptions().dtype(torch_type<T>::dtype).device(device()));
+        DeviceMatrixView<T> dL_dinput(batch_size, network_.get_input_width(), network_.get_input_width(),
+                                      get_dl_dinput ? reinterpret_cast<T *>(input_grad.data_ptr()) : nullptr);
+        network_.backward_pass_recompute(input_dm, dL_doutput, net_gradients_.GetViews(), get_dl_dinput ? &dL_dinput : nullptr);
+        return {input_grad, GradientsTensor(pack_transpose_gradient)};
+    }
+
+    bool can_train_with_encoding(const Module &encoding) const override {
+        const tnn_grid_desc *grid = encoding.grid_descriptor();
+        return grid && network_.supports_grid_input(*grid) && network_.supports_grid_training(*grid);
+    }
+
+    std::tuple<torch::Tensor, torch::Tensor> backward_with_encoding(const Module &encoding, const torch::Tensor &positions,
+                                                                    const torch::Tensor &grad_output, bool pack_transpose_gradient) override {
+        this->enter();
+        const tnn_grid_desc *grid = encoding.grid_descriptor();
+        if (!grid || !network_.supports_grid_training(*grid))
+            throw std::invalid_argument("backward_with_encoding: this encoding / network pair trains as two modules (" + std::string(tnn_last_error()) + ")");
+        CHECK_INPUT(positions);
+        TORCH_CHECK(positions.dim() == 2 && positions.scalar_type() == torch::kFloat32, "positions must be a float32 matrix");
+        if (positions.sizes()[1] != (int64_t)grid->n_dims) throw std::runtime_error("Input tensor has incorrect dimensions");
+        const size_t batch_size = positions.sizes()[0];
+        if (batch_size == 0 || batch_size % 8 != 0) throw std::invalid_argument("Batch size is not divisible by 8.");
+        CheckedGradOutput(grad_output, batch_size);
+        DeviceMatrixView<T> dL_doutput(batch_size, network_.get_output_width(), network_.get_output_width(), reinterpret_cast<T *>(grad_output.data_ptr()));
+        // the scatter overwrites its whole destination: it is the tensor that is handed back
+        torch::Tensor table_grad = torch::empty({(int64_t)tnn_grid_n_params(grid), 1}, torch::TensorOptions().dtype(torch::kFloat32).device(device()));
+        network_.backward_with_grid(*grid, encoding.grid_table(), positions.data_ptr<float>(), dL_doutput, net_gradients_.GetViews(),
+                                    table_grad.data_ptr<float>());
+        return {GradientsTensor(pack_transpose_gradient), table_grad};
+    }
+
     torch::Tensor initialize_params() override { return get_params(); }
     torch::Tensor get_params() override {
         this->enter();
@@ -459,6 +518,31 @@ template <typename T, int WIDTH> class NetworkModule : public Module {
                                         std::to_string(width));
         if (input_tensor.sizes()[0] % 8 != 0) throw std::invalid_argument("Batch size is not divisible by 8.");
         return input_tensor.sizes()[0];
+    }
+
+    void CheckedGradOutput(const torch::Tensor &grad_output, const size_t batch_size) const {
+        CHECK_INPUT(grad_output);
+        TORCH_CHECK(grad_output.dim() == 2, "grad_output must have two dimensions");
+        TORCH_CHECK(grad_output.scalar_type() == torch_type<T>::dtype, "grad_output has the wrong dtype");
+        if (grad_output.size(1) != network_.get_output_width())
+            throw std::invalid_argument("grad_output.size(1): " + std::to_string(grad_output.size(1)) +
+                                        " is not equal to  get_padded_output_width" + std::to_string(network_.get_output_width()));
+        if ((size_t)grad_output.size(0) != batch_size)
+            throw std::invalid_argument("grad_output has " + std::to_string(grad_output.size(0)) + " rows, the forward pass had " + std::to_string(batch_size));
+    }
+
+    /// The raw gradients the last backward pass left in net_gradients_, as a fresh tensor: a copy, or (packed) the output of the
+    /// pack-and-transpose kernel, which writes the tensor directly.
+    torch::Tensor GradientsTensor(const bool packed) {
+        const int64_t n = (int64_t)net_gradients_.nelements();
+        torch::Tensor out = torch::empty({n, 1}, torch::TensorOptions().dtype(torch_type<T>::dtype).device(device()));
+        if (packed)
+            tnn::abi_check(tnn_pack_and_transpose(tnn::dtype_of<T>::value, WIDTH, network_.get_n_hidden_layers() + 1, net_gradients_.data(), out.data_ptr(),
+                                                  this->get_queue().abi()));
+        else
+            tnn::hip_check(hipMemcpyAsync(out.data_ptr(), net_gradients_.data(), (size_t)n * sizeof(T), hipMemcpyDeviceToDevice, this->get_queue().get()),
+                           "hipMemcpyAsync");
+        return out;
     }
 
     DeviceMatricesView<T> ForwardViews(const size_t batch_size) const {

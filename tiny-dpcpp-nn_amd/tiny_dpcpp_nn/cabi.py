@@ -96,6 +96,18 @@ class Harness:
                                              int(dw_fp32), ptr(dX), M, ptr(ws), ws_bytes, self.stream()))
         return ib, dW, dX
 
+    def backward_recompute(self, desc, prep_fwd, prep_bwd, x_t, dLdy_t, want_dx=True, dw_fp32=True):
+        """Weight gradients (and dL/dx) for a given dL/dy with the forward pass formed again on chip (tnn_mlp_backward_recompute)."""
+        M, W = x_t.shape
+        n_mats = desc.n_hidden_layers + 1
+        ws_bytes = self.lib.tnn_mlp_train_step_workspace_bytes(ctypes.byref(desc), M)
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=self.dev)
+        dW = torch.full((n_mats, W, W), float("nan"), dtype=torch.float32 if dw_fp32 else x_t.dtype, device=self.dev)
+        dX = torch.full((M, W), float("nan"), dtype=x_t.dtype, device=self.dev) if want_dx else None
+        _lib.check(self.lib.tnn_mlp_backward_recompute(ctypes.byref(desc), ptr(prep_fwd), ptr(prep_bwd), ptr(x_t), ptr(dLdy_t), ptr(dW), int(dw_fp32),
+                                                       ptr(dX), M, ptr(ws), ws_bytes, self.stream()))
+        return dW, dX
+
     def l2_loss(self, dtype, pred_t, targets_t, loss_scale, want_values=True):
         n = pred_t.numel()
         values = torch.empty(pred_t.shape, dtype=torch.float32, device=self.dev) if want_values else None

@@ -76,7 +76,10 @@ class _NativeCall(torch.autograd.Function):
     @staticmethod
     def forward(ctx, owner, x, params):
         native = owner.tnn_module
-        y = native.fwd(x) if owner.training else native.inference(x)
+        # A network whose shape has the one-kernel backward pass keeps no activations: its training forward is the inference
+        # kernel, and the backward pass forms the activations again on chip from the saved input.
+        ctx.recompute = bool(owner._is_network and x.shape[0] > 0 and native.can_recompute_backward())
+        y = native.fwd(x) if (owner.training and not ctx.recompute) else native.inference(x)
         if x.shape[0] > 0:
             y = y.reshape(x.shape[0], -1)
         ctx.owner = owner
@@ -104,7 +107,10 @@ class _NativeCall(torch.autograd.Function):
             elif owner._is_network:
                 # weight gradients packed into the parameter layout; dL/dx costs a product with the first matrix and a
                 # batch-sized store, so it is asked for only when autograd wants it
-                dx, dparams = owner.tnn_module.bwd_no_encoding_grad(dy, True, bool(ctx.needs_input_grad[1]))
+                if ctx.recompute:
+                    dx, dparams = owner.tnn_module.bwd_recompute(dy, x, True, bool(ctx.needs_input_grad[1]))
+                else:
+                    dx, dparams = owner.tnn_module.bwd_no_encoding_grad(dy, True, bool(ctx.needs_input_grad[1]))
                 if dx is not None:
                     dx = dx.reshape(x.shape[0], -1)
             else:
@@ -117,6 +123,35 @@ class _NativeCall(torch.autograd.Function):
         if dx is not None and scale != 1.0:
             dx = dx / scale
         return None, dx, dparams
+
+
+class _EncodedNetworkCall(torch.autograd.Function):
+    """A grid encoding and its network as one call in both directions: the forward pass is the fused inference kernel (the
+    encoded matrix is never stored), the backward pass forms encoding and activations again on chip and returns the weight
+    gradients (packed layout) and the gradient of the table. Positions get no gradient, as in the reference
+    (dpcpp_bindings/tiny_dpcpp_nn/modules.py:114-128)."""
+
+    @staticmethod
+    def forward(ctx, owner, positions, net_params, table):
+        y = owner.network.tnn_module.inference_with_encoding(owner.encoding.tnn_module, positions)
+        ctx.owner = owner
+        ctx.save_for_backward(positions, net_params, table)
+        return y.reshape(positions.shape[0], -1)[:, : owner.n_output_dims]
+
+    @staticmethod
+    def backward(ctx, dy):
+        owner = ctx.owner
+        positions, net_params, table = ctx.saved_tensors
+        scale = owner.network.loss_scale
+        dy = F.pad(dy, [0, owner.width - dy.shape[1]]) if dy.shape[1] < owner.width else dy
+        if scale != 1.0:
+            dy = dy * scale
+        with torch.no_grad():
+            dnet, dtable = owner.network.tnn_module.bwd_with_encoding(owner.encoding.tnn_module, positions, dy.contiguous(), True)
+            if scale != 1.0:
+                dnet = dnet / scale
+                dtable = dtable / scale
+        return None, None, dnet.reshape(net_params.shape).to(net_params.dtype), dtable.reshape(table.shape).to(table.dtype)
 
 
 class Module(torch.nn.Module):
@@ -295,13 +330,27 @@ class NetworkWithInputEncoding(Module):
         self.network.set_params(params)
 
     def forward(self, x):
-        one_kernel = (not self.training and not torch.is_grad_enabled() and x.shape[0] > 0
-                      and self.network.tnn_module.can_fuse_encoding(self.encoding.tnn_module))
-        return self._fused_inference(x) if one_kernel else self.network_with_encoding(x)
+        if x.shape[0] == 0:
+            return self.network_with_encoding(x)
+        net, enc = self.network.tnn_module, self.encoding.tnn_module
+        if not torch.is_grad_enabled():
+            return self._fused_inference(x) if net.can_fuse_encoding(enc) else self.network_with_encoding(x)
+        if net.can_train_with_encoding(enc):
+            return self._fused_call(x)
+        return self.network_with_encoding(x)
+
+    def _fused_call(self, x):
+        """With autograd: one kernel forward (values as the two modules in turn), one kernel plus the scatter backward."""
+        batch = x.shape[0]
+        rows = _rows_padded(batch)
+        self.encoding._push_before_forward()
+        self.network._push_before_forward()
+        positions = _pad_rows(x.detach(), rows).to(torch.float32).contiguous()
+        return _EncodedNetworkCall.apply(self, positions, self.network.params, self.encoding.params)[:batch]
 
     def _fused_inference(self, x):
-        """Evaluation without autograd on a grid encoding: one kernel, the encoded matrix is never stored; the values are those
-        of the two modules in turn (the reference's only route)."""
+        """Without autograd on a grid encoding: one kernel, the encoded matrix is never stored; the values are those of the two
+        modules in turn (the reference's only route)."""
         batch = x.shape[0]
         rows = _rows_padded(batch)
         self.encoding._push_before_forward()

@@ -60,7 +60,7 @@ def parse():
     ap.add_argument("--reps", type=int, default=5, help="repetitions of --steps timed steps; the median is reported")
     ap.add_argument("--prewarm-ms", type=float, default=300.0,
                     help="untimed calls for this long before the declared warm-up (a fresh process starts at idle clocks)")
-    ap.add_argument("--workload", default="all", choices=["all", "train", "train_fb", "train_w128", "infer", "grid", "grid_mlp", "grid_train"])
+    ap.add_argument("--workload", default="all", choices=["all", "train", "train_fb", "train_w128", "infer", "grid", "grid_mlp", "grid_train", "py_infer", "py_train", "py_grid_train"])
     ap.add_argument("--batch-log2", type=int, default=None)
     ap.add_argument("--packed-scatter", action="store_true",
                     help="grid_train only: gradient table in fp16 with one packed atomic per feature pair (tnn_grid_backward_packed)")
@@ -68,6 +68,8 @@ def parse():
                     help="grid and grid_mlp: encode the points as they come instead of ordering the batch by cell in every step")
     ap.add_argument("--unfused", action="store_true",
                     help="grid_train: encoding, network step and scatter as three calls with the encoded matrix in memory")
+    ap.add_argument("--push-only-when-changed", action="store_true",
+                    help="py_* workloads: switch the modules' push of `params` before every forward off (push_params_every_forward = False)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-parity", action="store_true", help="skip the oracle check in front of the timing (profiling runs)")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -812,6 +814,133 @@ class Bench:
         return out, cfg, w
 
 
+# ------------------------------------------------------------------------------------------------------------------
+# The drop-in itself: tiny_dpcpp_nn.Network / NetworkWithInputEncoding with torch.optim.Adam, as a user of the reference's Python
+# package would run them (the reference's own figures of this kind: samples/benchmark_pytorch.py:24-198). Same shapes as the
+# C-ABI legs; each leg also times the C-ABI call that does the same work, in the same process, and reports the ratio.
+# ------------------------------------------------------------------------------------------------------------------
+def py_legs(b, which):
+    import torch
+
+    import tiny_dpcpp_nn as tcnn
+    args, t, lib = b.args, b.t, b.lib
+    from tiny_dpcpp_nn.cabi import ptr
+    dev = "cuda"
+    W = 64
+    net_cfg = lambda n_hidden: {"otype": "FullyFusedMLP", "activation": "ReLU", "output_activation": "None", "n_neurons": W, "n_hidden_layers": n_hidden}
+    every = not args.push_only_when_changed
+    push = "params pushed before every forward (the reference's behaviour)" if every else "params pushed only when they changed"
+
+    def timed(fn, steps=None):
+        return b.timer(steps).run(lambda i: fn())
+
+    if which == "py_infer":
+        M = 1 << (args.batch_log2 or 18)
+        net = tcnn.Network(W, W, net_cfg(4), dtype=torch.bfloat16, use_bias=False)
+        net.push_params_every_forward = every
+        net.eval()
+        x = (torch.rand((M, W), device=dev) * 2 - 1).to(torch.bfloat16)
+        with torch.no_grad():
+            y = net(x)
+            tm = timed(lambda: net(x))
+        c = b.mlp_case()
+        ref = b.leg_infer(c, M=M)
+        flops = 2 * M * W * W * 5
+        bytes_ = 2 * M * W * 2 + 5 * W * W * 2
+        ach = bytes_ / (tm["ms"] * 1e-3) / 1e9
+        roof = {"bound": "hbm", "achieved": ach, "peak": PEAK_HBM, "unit": "GB/s", "frac": ach / PEAK_HBM, "traffic": None,
+                "kernel": "whole Python call: Network.forward in eval mode under no_grad", "kernel_ms": tm["ms"], "algorithmic_bytes_per_launch": bytes_,
+                "mfma_frac": flops / (tm["ms"] * 1e-3) / 1e12 / PEAK_MFMA_BF16}
+        out = line(METRIC, "samples/s", "bf16", f"tiny_dpcpp_nn.Network inference from Python: w64, 4 hidden layers, bf16, batch 2^{M.bit_length() - 1}; {push}",
+                   M, tm, b.K, b.Wm, args, roof)
+        out.update({"c_abi_ms_per_step": ref["ms_per_step"], "ratio_to_c_abi": tm["ms"] / ref["ms_per_step"], "output_shape": list(y.shape)})
+        return out
+
+    if which == "py_train":
+        M = 1 << (args.batch_log2 or 18)
+        net = tcnn.Network(W, W, net_cfg(4), dtype=torch.bfloat16, use_bias=False)
+        net.push_params_every_forward = every
+        net.train()
+        opt = torch.optim.Adam(net.parameters(), lr=1e-3, betas=(0.9, 0.99), eps=1e-15)
+        x = (torch.rand((M, W), device=dev) * 2 - 1).to(torch.bfloat16)
+        targets = torch.rand((M, W), device=dev)
+        losses = []
+
+        def step():
+            opt.zero_grad(set_to_none=True)
+            loss = torch.nn.functional.mse_loss(net(x).float(), targets)
+            loss.backward()
+            opt.step()
+            return loss
+
+        losses.append(float(step().detach()))
+        tm = timed(step)
+        losses.append(float(step().detach()))
+        # the module's own share of that step: forward and backward for a dL/dy that is already there (no loss and no optimizer
+        # kernels of PyTorch's: its mse_loss alone reads and writes five batch-sized fp32 matrices)
+        dy = (torch.rand((M, W), device=dev) / M).to(torch.bfloat16)
+
+        def forward_backward():
+            net.params.grad = None
+            net(x).backward(dy)
+
+        tm_fb = timed(forward_backward)
+        # ... and the same step with PyTorch's one-kernel Adam (fused=True), where the optimizer is one launch instead of a dozen
+        opt = torch.optim.Adam(net.parameters(), lr=1e-3, betas=(0.9, 0.99), eps=1e-15, fused=True)
+        tm_fused_adam = timed(step)
+        c = b.mlp_case()
+        ref = b.leg_train(c, torch.rand((c["M"], W), device=t.dev, generator=c["gen"]))
+        flops = 3 * 2 * M * W * W * 5
+        ach = flops / (tm["ms"] * 1e-3) / 1e12
+        roof = {"bound": "mfma", "achieved": ach, "peak": PEAK_MFMA_BF16, "unit": "TFLOP/s", "frac": ach / PEAK_MFMA_BF16, "traffic": None,
+                "kernel": "whole Python step: Network.forward, torch mse_loss, backward (weight gradients with the activations formed again on chip), "
+                          "torch.optim.Adam", "kernel_ms": tm["ms"], "algorithmic_flops_per_launch": flops}
+        out = line(METRIC, "samples/s", "bf16",
+                   f"tiny_dpcpp_nn.Network training step from Python with torch.optim.Adam: w64, 4 hidden layers, bf16, batch 2^{M.bit_length() - 1}, "
+                   f"mse_loss in PyTorch; {push}", M, tm, b.K, b.Wm, args, roof)
+        out.update({"c_abi_ms_per_step": ref["ms_per_step"], "ratio_to_c_abi": tm["ms"] / ref["ms_per_step"], "loss_first": losses[0], "loss_last": losses[1],
+                    "module_forward_backward_ms": tm_fb["ms"], "module_forward_backward_ratio_to_c_abi": tm_fb["ms"] / ref["ms_per_step"],
+                    "ms_per_step_with_fused_torch_adam": tm_fused_adam["ms"],
+                    "note": "the C-ABI step computes the L2 loss and Adam inside its two kernels; here PyTorch computes them: mse_loss forward and "
+                            "backward on a 2^18 x 64 fp32 matrix (about 105 us of its kernels) and torch.optim.Adam (about 45 us of small launches)"})
+        return out
+
+    # py_grid_train: BASELINE config 4 through NetworkWithInputEncoding
+    M = 1 << (args.batch_log2 or 18)
+    enc_cfg = {"otype": "HashGrid", "type": "Hash", "n_levels": 16, "n_features_per_level": 2, "log2_hashmap_size": 19, "base_resolution": 16,
+               "per_level_scale": 1.5}
+    model = tcnn.NetworkWithInputEncoding(2, 3, net_cfg(2), enc_cfg, dtype=torch.float16, use_bias=False)
+    model.network.push_params_every_forward = every
+    model.encoding.push_params_every_forward = every
+    model.train()
+    opt = torch.optim.Adam(model.parameters(), lr=1e-3, betas=(0.9, 0.99), eps=1e-15)
+    x = torch.rand((M, 2), device=dev)
+    targets = torch.rand((M, 3), device=dev)
+
+    def step():
+        opt.zero_grad(set_to_none=True)
+        loss = torch.nn.functional.mse_loss(model(x).float(), targets)
+        loss.backward()
+        opt.step()
+        return loss
+
+    K, Wm = min(b.K, 50), min(b.Wm, 5)
+    first = float(step().detach())
+    tm = b.timer(K, Wm).run(lambda i: step())
+    last = float(step().detach())
+    ref, _, _ = b.leg_grid_train()
+    bpp = 8 + 32 * 2 + 16 * 4 * 2 * 4 * 2  # the scatter's algorithmic bytes per point, as in the grid_train leg
+    ach = bpp * M / (tm["ms"] * 1e-3) / 1e9
+    roof = {"bound": "hbm", "achieved": ach, "peak": PEAK_HBM, "unit": "GB/s", "frac": ach / PEAK_HBM, "traffic": None,
+            "kernel": "whole Python step: fused encoding + network forward, torch mse_loss, fused backward + scatter, torch.optim.Adam over "
+                      "network and table", "kernel_ms": tm["ms"], "algorithmic_bytes_per_launch": bpp * M}
+    out = line("hash-grid + fused-MLP training samples/s (2-D, 16x2, log2 19; w64, 2 hidden layers; batch 2^18; whole step with both Adam updates)",
+               "samples/s", "f16", f"tiny_dpcpp_nn.NetworkWithInputEncoding training step from Python with torch.optim.Adam (BASELINE config 4), "
+               f"2^{M.bit_length() - 1} points; {push}", M, tm, K, Wm, args, roof)
+    out.update({"c_abi_ms_per_step": ref["ms_per_step"], "ratio_to_c_abi": tm["ms"] / ref["ms_per_step"], "loss_first": first, "loss_last": last})
+    return out
+
+
 def sub(leg):
     """A leg as a sub-object of the default line: the fields that differ from the top level."""
     keep = ("value", "unit", "ms_per_step", "ms_per_step_reps", "steps", "warmup", "dtype", "config", "roofline", "mfma_frac", "parity_checked",
@@ -889,6 +1018,9 @@ def main():
         out, cfg, w = b.leg_grid_train()
         if do_cpu:
             out["cpu_baseline"] = cpu_baseline_grid_train(oracle, cfg, oracle.round(w, FP16))
+
+    if wl in ("py_infer", "py_train", "py_grid_train"):
+        out = py_legs(b, wl)
 
     if args.copy_calibration:
         from tiny_dpcpp_nn.cabi import ptr

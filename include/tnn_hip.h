@@ -112,6 +112,15 @@ int tnn_pack_and_transpose(int dtype, int width, int n_mats, const void *d_raw, 
 int tnn_zero_weights_padding(const tnn_mlp_desc *desc, void *d_packed, int unpadded_input_width,
                              int unpadded_output_width, int use_bias, tnn_stream_t stream);
 
+/* Network::set_weights_matrices for parameters that are already packed and on the device (include/network/Network.h:90-112
+ * with ZeroWeightsPadding :171-233 and TransposeWeights :235-238), in one launch: d_src_packed (src_dtype: T or fp32
+ * masters, rounded to T) -> the packed copy in T with the padding weights zeroed, its packed transpose, and both prepared
+ * operand sets. Bit for bit what tnn_cast + tnn_zero_weights_padding + tnn_packed_transpose + tnn_mlp_prepare_weights give;
+ * it is what a module runs in front of every forward pass (dpcpp_bindings/tiny_dpcpp_nn/modules.py:253). */
+int tnn_mlp_set_packed_weights(const tnn_mlp_desc *desc, const void *d_src_packed, int src_dtype, int unpadded_input_width,
+                               int unpadded_output_width, int use_bias, void *d_packed_T, void *d_packed_transposed_T,
+                               void *d_prepared_fwd, void *d_prepared_bwd, tnn_stream_t stream);
+
 /* Bytes of ONE prepared buffer (forward and backward operand sets have the same size). */
 size_t tnn_mlp_prepared_bytes(const tnn_mlp_desc *desc);
 /* Packed parameters (type T, or fp32 master weights when src_is_fp32 != 0; they are rounded to T) ->

@@ -69,7 +69,7 @@ def test_default_run_carries_the_whole_metric():
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("workload", ["train", "train_fb", "infer", "grid", "grid_mlp", "grid_train"])
+@pytest.mark.parametrize("workload", ["train", "train_fb", "infer", "grid", "grid_mlp", "grid_train", "py_infer", "py_train", "py_grid_train"])
 def test_every_workload_prints_the_contract_line(workload):
     r = subprocess.run([sys.executable, BENCH, "--workload", workload, "--steps", "5", "--warmup", "2", "--reps", "2", "--prewarm-ms", "20",
                         "--no-cpu-baseline"], capture_output=True, text=True, timeout=600)
@@ -82,3 +82,5 @@ def test_every_workload_prints_the_contract_line(workload):
     check_roofline(out["roofline"])
     assert out["n_gpus"] == 1 and out["vs_baseline"] is None and out["data"] == "synthetic"
     assert "workload" in out["config"] and out["value"] > 0
+    if workload.startswith("py_"):  # the drop-in's own legs carry the C-ABI call of the same work, timed in the same process
+        assert out["c_abi_ms_per_step"] > 0 and abs(out["ratio_to_c_abi"] - out["ms_per_step"] / out["c_abi_ms_per_step"]) < 1e-9

@@ -4,7 +4,7 @@ import ctypes
 import numpy as np
 import pytest
 
-from tolerances import BF16, FP16, PROPAGATED, assert_close, assert_propagated, max_norm_rel
+from tolerances import BF16, FP16, FP32, PROPAGATED, assert_close, assert_propagated, max_norm_rel
 
 pytestmark = pytest.mark.gpu
 
@@ -51,6 +51,16 @@ def test_prepare_and_layout_kernels_bit_exact(tnn, oracle):
                 z = packed.clone()
                 _lib.check(tnn.lib.tnn_zero_weights_padding(ctypes.byref(desc), ptr(z), n_in, n_out, int(bias), tnn.stream()))
                 assert np.array_equal(tnn.host(z), oracle.zero_weights_padding(oracle.pack_weights(w, n_mats, W), n_mats, W, n_in, n_out, bias))
+                # the one-launch route of a module's push: the same four copies as cast + zero padding + packed transpose + prepare
+                zt = torch.empty_like(z)
+                _lib.check(tnn.lib.tnn_packed_transpose(dtype, W, n_mats, ptr(z), ptr(zt), tnn.stream()))
+                pf, pb = tnn.prepare_packed(desc, z)
+                for src in (packed, packed.float()):
+                    outs = [torch.full_like(t, float("nan")) for t in (z, zt, pf, pb)]
+                    _lib.check(tnn.lib.tnn_mlp_set_packed_weights(ctypes.byref(desc), ptr(src), FP32 if src.dtype == torch.float32 else dtype, n_in, n_out,
+                                                                  int(bias), ptr(outs[0]), ptr(outs[1]), ptr(outs[2]), ptr(outs[3]), tnn.stream()))
+                    for got, want in zip(outs, (z, zt, pf, pb)):
+                        assert torch.equal(got.view(torch.int16), want.view(torch.int16))
 
 
 @pytest.mark.parametrize("dtype", [BF16, FP16])

@@ -537,6 +537,17 @@ def test_params_data_assignment_reaches_the_kernels(tcnn):
         # every weight 1/32, no activation: column sums of x over the 8 real inputs, then 32 * (1/32) per later matrix
         expect = (x.to(torch.bfloat16).float().sum(1, keepdim=True) / 32).expand(-1, 4)
         assert torch.allclose(y.float(), expect, rtol=2e-2, atol=1e-3)
+    # an encoding's table is the tensor itself (no copy is pushed): a write through .data is seen by the next forward
+    enc = tcnn.Encoding(2, dict(GRID_2D))
+    pts2 = torch.rand((64, 2), device=DEVICE)
+    enc.params.data[:] = 0.25
+    with torch.no_grad():
+        e = enc(pts2)
+    assert torch.allclose(e[:, :32], torch.full_like(e[:, :32], 0.25), atol=1e-6)   # the corner weights of a cell sum to one
+    enc.params.data[:] = 0.0
+    with torch.no_grad():
+        assert float(enc(pts2).abs().max()) == 0.0
+    assert float(enc.get_params().abs().max()) == 0.0 and enc.get_params().data_ptr() != enc.params.data_ptr()
     # the fused encoding + network route reads both modules' parameters the same way
     nwe = tcnn.NetworkWithInputEncoding(2, 3, net_config(64, 2), dict(GRID_2D), dtype=torch.float16)
     nwe.eval()

@@ -829,9 +829,79 @@ static int check_batch(size_t M) {
     return TNN_OK;
 }
 
+// Everything Network::set_weights_matrices derives from packed parameters, in one pass: the packed copy in T with the
+// weights that only see padding zeroed, its packed transpose, and both operand-order copies. A thread takes one slot of the
+// operand-order index space (which covers every matrix element once, plus the empty half-tile at width 16).
+template <typename T, typename SRC>
+__global__ void set_packed_weights_kernel(const SRC *__restrict__ src, T *__restrict__ packed, T *__restrict__ packed_t, T *__restrict__ fwd,
+                                          T *__restrict__ bwd, int W, int n_mats, int live_in, int live_out) {
+    const int NI = (W + 31) / 32, NK = W / 16;
+    const int per_mat = NI * NK * 512;
+    const int total = n_mats * per_mat;
+    for (int idx = blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += gridDim.x * blockDim.x) {
+        const int l = idx / per_mat;
+        int r = idx % per_mat;
+        const int t = r & 7;
+        const int lane = (r >> 3) & 63;
+        r >>= 9;
+        const int kb = r % NK, a = r / NK;
+        const int h = lane >> 5, i = lane & 31;
+        const int outer = 32 * a + swap23(i), inner = 16 * kb + 8 * h + t;
+        T vf = (T)0.0f, vb = (T)0.0f;
+        if (outer < W) {
+            const size_t m = (size_t)l * W * W;
+            // rows of the first matrix from live_in on and columns of the last matrix from live_out on only see padding
+            auto weight = [&](int k, int n) { return ((l == 0 && k >= live_in) || (l == n_mats - 1 && n >= live_out)) ? (T)0.0f : (T)(float)src[m + packed_coord(k, n, W)]; };
+            vf = weight(inner, outer);
+            vb = weight(outer, inner);
+            packed[m + packed_coord(inner, outer, W)] = vf;
+            packed_t[m + packed_coord(outer, inner, W)] = vf; // element (k, n) of W is element (n, k) of its transpose
+        }
+        fwd[idx] = vf;
+        bwd[idx] = vb;
+    }
+}
+
 } // namespace tnn
 
 using namespace tnn;
+
+TNN_API int tnn_mlp_set_packed_weights(const tnn_mlp_desc *desc, const void *d_src_packed, int src_dtype, int unpadded_input_width,
+                                       int unpadded_output_width, int use_bias, void *d_packed_T, void *d_packed_transposed_T,
+                                       void *d_prepared_fwd, void *d_prepared_bwd, tnn_stream_t stream) {
+    int rc = check_mlp_desc(desc);
+    if (rc) return rc;
+    if (!d_src_packed || !d_packed_T || !d_packed_transposed_T || !d_prepared_fwd || !d_prepared_bwd)
+        return fail(TNN_ERR_INVALID_ARGUMENT, "NULL pointer argument");
+    if (d_src_packed == d_packed_T || d_src_packed == d_packed_transposed_T) return fail(TNN_ERR_INVALID_ARGUMENT, "the source must not be one of the destinations");
+    const int W = desc->width;
+    if (unpadded_input_width > W || unpadded_output_width > W || unpadded_input_width <= 0 || unpadded_output_width <= 0)
+        return fail(TNN_ERR_INVALID_ARGUMENT, "Padded weights width cannot be less than the unpadded.");
+    // include/network/Network.h:191-202: with the bias trick the ones reach up to the next multiple of 16, and an input width
+    // that already is one leaves the whole padded width live
+    const int live_in = !use_bias ? unpadded_input_width : (unpadded_input_width % 16 == 0 ? W : (unpadded_input_width / 16 + 1) * 16);
+    if (live_in > W) return fail(TNN_ERR_INVALID_ARGUMENT, "one_padded_input_width > padded_input_width, the input width is too small.");
+    const int n_mats = desc->n_hidden_layers + 1;
+    const int total = (int)prepared_elems(desc);
+    const int blocks = (total + 255) / 256;
+    hipStream_t s = as_stream(stream);
+#define TNN_SPW(T_, S_)                                                                                                                          \
+    TNN_LAUNCH((set_packed_weights_kernel<T_, S_>), dim3(blocks), dim3(256), 0, s, (const S_ *)d_src_packed, (T_ *)d_packed_T, (T_ *)d_packed_transposed_T, \
+               (T_ *)d_prepared_fwd, (T_ *)d_prepared_bwd, W, n_mats, live_in, unpadded_output_width)
+    if (desc->dtype == TNN_BF16) {
+        if (src_dtype == TNN_FP32) TNN_SPW(bf16_t, float);
+        else if (src_dtype == TNN_BF16) TNN_SPW(bf16_t, bf16_t);
+        else if (src_dtype == TNN_FP16) TNN_SPW(bf16_t, fp16_t);
+        else return fail(TNN_ERR_UNSUPPORTED, "src_dtype %d", src_dtype);
+    } else {
+        if (src_dtype == TNN_FP32) TNN_SPW(fp16_t, float);
+        else if (src_dtype == TNN_BF16) TNN_SPW(fp16_t, bf16_t);
+        else if (src_dtype == TNN_FP16) TNN_SPW(fp16_t, fp16_t);
+        else return fail(TNN_ERR_UNSUPPORTED, "src_dtype %d", src_dtype);
+    }
+#undef TNN_SPW
+    return check_launch("set_packed_weights_kernel");
+}
 
 TNN_API size_t tnn_mlp_prepared_bytes(const tnn_mlp_desc *desc) {
     if (check_mlp_desc(desc)) return 0;

@@ -88,12 +88,14 @@ template <typename T, MatrixLayout _layout = MatrixLayout::RowMajor> class Devic
   public:
     DeviceMatrix(const size_t m, const size_t n, tnn::queue &stream)
         : m_rows(m), m_cols(n), m_q(stream), m_data(tnn::detail::device_alloc<T>(m * n)) {}
+    /// A matrix over device memory that somebody else owns (a PyTorch tensor, say) and keeps alive; nothing is freed here.
+    DeviceMatrix(const size_t m, const size_t n, tnn::queue &stream, T *borrowed) : m_rows(m), m_cols(n), m_q(stream), m_data(borrowed), m_owns(false) {}
     DeviceMatrix() = delete;
     DeviceMatrix(const DeviceMatrix &other) : m_rows(other.m_rows), m_cols(other.m_cols), m_q(other.m_q), m_data(tnn::detail::device_alloc<T>(other.n_elements())) {
         tnn::hip_check(hipMemcpyAsync(m_data, other.m_data, n_bytes(), hipMemcpyDeviceToDevice, m_q.get()), "hipMemcpyAsync");
         m_q.wait();
     }
-    DeviceMatrix(DeviceMatrix &&other) : m_rows(other.m_rows), m_cols(other.m_cols), m_q(other.m_q), m_data(other.m_data) { other.m_data = nullptr; }
+    DeviceMatrix(DeviceMatrix &&other) : m_rows(other.m_rows), m_cols(other.m_cols), m_q(other.m_q), m_data(other.m_data), m_owns(other.m_owns) { other.m_data = nullptr; }
     DeviceMatrix &operator=(const DeviceMatrix &other) {
         if (this == &other) return *this;
         if (other.m_rows != m_rows || other.m_cols != m_cols) throw std::invalid_argument("Cannot assign matrices of differing dimensions.");
@@ -101,7 +103,9 @@ template <typename T, MatrixLayout _layout = MatrixLayout::RowMajor> class Devic
         m_q.wait();
         return *this;
     }
-    ~DeviceMatrix() { tnn::detail::device_free(m_data); }
+    ~DeviceMatrix() {
+        if (m_owns) tnn::detail::device_free(m_data);
+    }
 
     tnn::event fill(const T val) {
         tnn::abi_check(tnn_fill(tnn::dtype_of<T>::value, m_data, n_elements(), (float)val, m_q.abi()));
@@ -159,6 +163,7 @@ template <typename T, MatrixLayout _layout = MatrixLayout::RowMajor> class Devic
     size_t m_rows, m_cols;
     tnn::queue &m_q;
     T *m_data;
+    bool m_owns = true;
 };
 
 template <typename T> class DeviceMatrices {

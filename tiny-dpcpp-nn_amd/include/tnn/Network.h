@@ -82,8 +82,11 @@ template <typename T> class Network : public NetworkBase<T> {
     template <typename Ts> void set_weights_matrices_from_device(Ts const *const d_weights, const bool weights_are_packed) {
         const int dtype = tnn::dtype_of<T>::value;
         const size_t n = m_weights_matrices.nelements();
-        if (weights_are_packed) {
-            tnn::abi_check(tnn_cast(dtype, m_weights_matrices.data(), tnn::dtype_of<Ts>::value, d_weights, n, m_q.abi()));
+        if (weights_are_packed) { // the route of every forward pass of a Python module: one launch for all four copies
+            const tnn_mlp_desc d = weights_desc();
+            tnn::abi_check(tnn_mlp_set_packed_weights(&d, d_weights, tnn::dtype_of<Ts>::value, (int)shape_.raw_in, (int)shape_.raw_out, shape_.bias ? 1 : 0,
+                                                      m_weights_matrices.data(), m_weightsT_matrices.data(), prepared_fwd_, prepared_bwd_, m_q.abi()));
+            return;
         } else { // the transposed copy is rebuilt below; until then it is the staging buffer of the converted values
             tnn::abi_check(tnn_cast(dtype, m_weightsT_matrices.data(), tnn::dtype_of<Ts>::value, d_weights, n, m_q.abi()));
             tnn::abi_check(tnn_pack_weights(dtype, shape_.width, shape_.hidden + 1, m_weightsT_matrices.data(), m_weights_matrices.data(), m_q.abi()));
@@ -129,7 +132,6 @@ template <typename T> class Network : public NetworkBase<T> {
         int hidden = 0, width = 0;
         uint32_t in = 0, out = 0;         // as the kernels see them: padded to the network width
         uint32_t raw_in = 0, raw_out = 0; // as the caller gave them
-        uint32_t live_in = 0;             // rows of the first matrix that see data: raw_in, or its next multiple of 16 with use_bias
         bool bias = false;
 
         static uint32_t round_up(const int value, const int multiple_of, const char *what) {
@@ -156,14 +158,12 @@ template <typename T> class Network : public NetworkBase<T> {
                                          ") is not supported: it must not exceed the network width " + std::to_string(network_width) + ".");
             if (n_hidden_layers < 1)
                 throw std::runtime_error("N hidden layers is " + std::to_string(n_hidden_layers) + " but must be >= 1, i.e., 1 hidden layer and 1 output layer.");
-            s.live_in = use_bias ? round_up(input_width, 16, "Input") : s.raw_in;
-            if (s.live_in > s.in) throw std::invalid_argument("the input width rounded up to 16 exceeds the padded input width.");
             s.bias = use_bias;
             return s;
         }
     };
 
-    /// After the packed weights changed: zero what only sees padding (rows of the first matrix from live_in on, columns of
+    /// After the packed weights changed: zero what only sees padding (rows of the first matrix that only see padding, columns of
     /// the last matrix from the caller's output width on; Network.h:171-233 of the reference), then rebuild the transposed
     /// packed copy and the two operand-order copies the kernels read. All on the network's stream.
     void finish_weights(const bool wait) {

@@ -61,6 +61,11 @@ template <typename T> class Encoding {
 
     /// The parameters of the encoding (null for encodings without any). Owned by the encoding.
     std::shared_ptr<DeviceMatrix<T>> get_params() const { return m_params; }
+    /// The encoding reads (and its owner trains) its parameters where `params` lies from now on; same number of elements.
+    void adopt_params(std::shared_ptr<DeviceMatrix<T>> params) {
+        if (!m_params || !params || params->size() != m_params->size()) throw std::invalid_argument("adopt_params: wrong number of parameters");
+        m_params = std::move(params);
+    }
     uint32_t get_input_width() const { return m_input_width; }
     uint32_t get_padded_output_width() const { return m_padded_output_width; }
     uint32_t get_output_width() const { return m_output_width; }

@@ -229,7 +229,13 @@ template <typename T> class EncodingModule : public Module {
         TORCH_CHECK((size_t)params.numel() == encoding_->get_n_params(), "params has ", params.numel(), " elements, the encoding has ",
                     encoding_->get_n_params());
         TORCH_CHECK(params.scalar_type() == torch_type<T>::dtype, "params has the wrong dtype");
-        encoding_->get_params()->copy_from_device(params.data_ptr<T>());
+        // No copy: from now on the table IS the caller's tensor (a reference keeps it alive), so later writes to it by any
+        // route are seen by the kernels, and pushing the same tensor again costs nothing. The reference copies, through the
+        // host (include/tnn_api.h:430-446); get_params() hands back a copy either way.
+        if (!table_alias_.defined() || table_alias_.data_ptr() != params.data_ptr()) {
+            encoding_->adopt_params(std::make_shared<DeviceMatrix<T>>(encoding_->get_n_params(), 1, this->get_queue(), params.data_ptr<T>()));
+            table_alias_ = params;
+        }
     }
 
     torch::Tensor get_params() override {
@@ -272,6 +278,7 @@ template <typename T> class EncodingModule : public Module {
     void initialize_ptr() {}
 
     std::shared_ptr<Encoding<T>> encoding_;
+    torch::Tensor table_alias_; // the tensor whose memory is the encoding's table, once set_params has been called
     torch::Tensor last_gradients_;
     size_t max_batch_size_; // the workspace fits every batch size seen so far
     T *output_encoding_ptr_;

@@ -80,12 +80,9 @@ class _NativeCall(torch.autograd.Function):
         # kernel, and the backward pass forms the activations again on chip from the saved input.
         ctx.recompute = bool(owner._is_network and x.shape[0] > 0 and native.can_recompute_backward())
         y = native.fwd(x) if (owner.training and not ctx.recompute) else native.inference(x)
-        if x.shape[0] > 0:
-            y = y.reshape(x.shape[0], -1)
         ctx.owner = owner
         ctx.save_for_backward(x, params)
-        visible = owner._visible_output_columns()
-        return y if visible is None else y[..., :visible]  # the rest of a network's output row is padding
+        return owner._visible_part(y, x.shape[0])
 
     @staticmethod
     def backward(ctx, dy):
@@ -187,6 +184,14 @@ class Module(torch.nn.Module):
     def _visible_output_columns(self):
         return None
 
+    def _visible_part(self, y, rows):
+        """The native module's result as [rows, visible columns]; no view is made when it already is that (a slice that keeps
+        everything still costs autograd a batch-sized zero fill and a copy on the way back)."""
+        if rows > 0 and y.dim() != 2:
+            y = y.reshape(rows, -1)
+        visible = self._visible_output_columns()
+        return y if (visible is None or visible == y.shape[-1]) else y[..., :visible]  # the rest of a network's output row is padding
+
     def _native_output_columns(self):
         return None
 
@@ -237,8 +242,12 @@ class Module(torch.nn.Module):
     def forward(self, x):
         batch = x.shape[0]
         self._push_before_forward()
-        y = _NativeCall.apply(self, self._prepare_input(x).contiguous(), self.params)
-        return y[:batch]
+        xin = self._prepare_input(x).contiguous()
+        if torch.is_grad_enabled():
+            y = _NativeCall.apply(self, xin, self.params)
+        else:  # nothing to record: straight to the kernel
+            y = self._visible_part(self.tnn_module.inference(xin), xin.shape[0])
+        return y if xin.shape[0] == batch else y[:batch]
 
 
 class Network(Module):

@@ -60,7 +60,7 @@ def parse():
     ap.add_argument("--reps", type=int, default=5, help="repetitions of --steps timed steps; the median is reported")
     ap.add_argument("--prewarm-ms", type=float, default=300.0,
                     help="untimed calls for this long before the declared warm-up (a fresh process starts at idle clocks)")
-    ap.add_argument("--workload", default="all", choices=["all", "train", "train_fb", "train_w128", "infer", "grid", "grid_mlp", "grid_train", "py_infer", "py_train", "py_grid_train"])
+    ap.add_argument("--workload", default="all", choices=["all", "train", "train_fb", "train_w128", "infer", "grid", "grid_mlp", "grid_train", "py_infer", "py_train", "py_grid_train", "line_probe"])
     ap.add_argument("--batch-log2", type=int, default=None)
     ap.add_argument("--packed-scatter", action="store_true",
                     help="grid_train only: gradient table in fp16 with one packed atomic per feature pair (tnn_grid_backward_packed)")
@@ -941,6 +941,46 @@ def py_legs(b, which):
     return out
 
 
+def line_probe(b):
+    """The ceiling for config 5's gather: random whole 128-byte lines read from buffers of several sizes (one that fits the
+    256 MB cache in front of the HBM several times over, the table's own 162 MiB, and 2 GiB, which fits nothing) by 2^21 threads
+    reading 32 lines each -- config 5's batch, and the 27-28 lines a point of that batch costs after the cell ordering. Nothing
+    but the loads is in the kernel (tnn_probe_line_gather)."""
+    import statistics
+
+    torch, t, lib, args = b.torch, b.t, b.lib, b.args
+    from tiny_dpcpp_nn.cabi import ptr
+    n_threads, per_thread = 1 << (args.batch_log2 or 21), 32
+    sink = torch.empty(n_threads, dtype=torch.int32, device=t.dev)
+    s = t.stream()
+    sizes = {"32 MiB": 32 << 20, "162 MiB (config 5's table)": 42519264 * 2 * 2, "2 GiB": 2 << 30}
+    res = {}
+    for name, nbytes in sizes.items():
+        buf = torch.zeros(nbytes // 4, dtype=torch.int32, device=t.dev)
+        n = [0]
+
+        def call(i):
+            n[0] += 1
+            if lib.tnn_probe_line_gather(ptr(buf), nbytes, n_threads, per_thread, n[0], ptr(sink), s):
+                raise RuntimeError(lib.tnn_last_error())
+
+        tm = b.timer(min(b.K, 50), min(b.Wm, 5)).run(call)
+        lines = n_threads * per_thread
+        res[name] = {"ms": tm["ms"], "lines_per_s": lines / (tm["ms"] * 1e-3), "bytes_of_lines_per_s": lines * 128 / (tm["ms"] * 1e-3)}
+        del buf
+        torch.cuda.empty_cache()
+    key = "162 MiB (config 5's table)"
+    ach = res[key]["bytes_of_lines_per_s"] / 1e9
+    tm = {"ms": res[key]["ms"], "reps_ms": [res[key]["ms"]], "wall_ms": res[key]["ms"]}
+    roof = {"bound": "hbm", "achieved": ach, "peak": PEAK_HBM, "unit": "GB/s", "frac": ach / PEAK_HBM, "traffic": n_threads * per_thread * 128,
+            "kernel": "line_gather_probe_kernel (random 128-byte lines, 32 in flight per thread, read-only)", "kernel_ms": res[key]["ms"],
+            "algorithmic_bytes_per_launch": n_threads * per_thread * 128}
+    out = line("random 128-byte line gathers per second (the ceiling of config 5's hash-grid gather)", "lines/s", "u32",
+               f"2^{n_threads.bit_length() - 1} threads x {per_thread} random lines of a buffer", n_threads * per_thread, tm, min(b.K, 50), min(b.Wm, 5), args, roof)
+    out["by_buffer_size"] = res
+    return out
+
+
 def sub(leg):
     """A leg as a sub-object of the default line: the fields that differ from the top level."""
     keep = ("value", "unit", "ms_per_step", "ms_per_step_reps", "steps", "warmup", "dtype", "config", "roofline", "mfma_frac", "parity_checked",
@@ -1021,6 +1061,8 @@ def main():
 
     if wl in ("py_infer", "py_train", "py_grid_train"):
         out = py_legs(b, wl)
+    if wl == "line_probe":
+        out = line_probe(b)
 
     if args.copy_calibration:
         from tiny_dpcpp_nn.cabi import ptr

@@ -437,6 +437,15 @@ int tnn_frequency_backward(const void *d_dLdy, int dy_dtype, uint32_t padded_wid
 int tnn_sh_forward(const float *d_x, uint32_t degree, void *d_out, int out_dtype, uint32_t padded_width, size_t M,
                    tnn_stream_t stream);
 
+/* Measurement aid, no counterpart in the reference: the rate at which the memory system serves the access pattern that
+ * bounds the hash-grid gather (include/encodings/grid.h:95-129 over a table beyond the caches), with nothing else in the
+ * kernel. n_threads threads (one per "point", workgroups of 256 as the encoding kernel's) each read 4 bytes from
+ * lines_per_thread (a multiple of 32) random 128-byte lines of d_buffer, 32 of them in flight at a time, and write one 4-byte
+ * sum to d_sink (n_threads x 4 bytes). The lines per second it reaches over a buffer of the table's size are the ceiling
+ * against which the encoding kernel's own line rate is read (bench.py --workload line_probe). */
+int tnn_probe_line_gather(const void *d_buffer, size_t buffer_bytes, size_t n_threads, int lines_per_thread, uint32_t seed, void *d_sink,
+                          tnn_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -91,6 +91,7 @@ SIGNATURES = {
     "tnn_grid_mlp_backward": (c_int, [ctypes.POINTER(GridDesc), ctypes.POINTER(MlpDesc), c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                       c_void_p, c_int, c_void_p, c_int, c_size_t, c_void_p, c_size_t, c_void_p]),
     "tnn_mlp_set_packed_weights": (c_int, [ctypes.POINTER(MlpDesc), c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
+    "tnn_probe_line_gather": (c_int, [c_void_p, c_size_t, c_size_t, c_int, ctypes.c_uint32, c_void_p, c_void_p]),
     "tnn_debug_set_meeting_spin_limit": (c_int, [c_int, ctypes.POINTER(c_int)]),
     "tnn_mlp_train_step_l2_static_max_bytes": (c_size_t, []),
     "tnn_mlp_train_step_l2_static": (

@@ -423,6 +423,50 @@ def test_network_with_grid_encoding_trains_through_one_kernel(tcnn, oracle, dtyp
     assert xg.grad is None
 
 
+def test_fused_training_route_at_a_batch_that_is_visited_in_cell_order(tcnn):
+    """From 2^17 rows on the fused backward pass visits the points in cell order (its tiles then hold other rows than the batch's,
+    and the order differs from run to run): sums over the batch agree with the two-module route to fp32 rounding, the per-row
+    output bit for bit. BASELINE config 4's shapes (2-D, 16 x 2, log2 19, w64 with 2 hidden layers, 3 outputs), half its batch."""
+    torch.manual_seed(23)
+    grid = {"otype": "HashGrid", "n_levels": 16, "n_features_per_level": 2, "log2_hashmap_size": 19, "base_resolution": 16, "per_level_scale": 1.5}
+    model = tcnn.NetworkWithInputEncoding(2, 3, net_config(64, 2), grid, dtype=torch.float16, use_bias=False)
+    with torch.no_grad():
+        model.encoding.params.copy_(torch.rand_like(model.encoding.params) * 2 - 1)
+    model.train()
+    batch = (1 << 17) + 8
+    x = torch.rand((batch, 2), device=DEVICE)
+    target = torch.rand((batch, 3), device=DEVICE)
+
+    def grads(run):
+        model.zero_grad(set_to_none=True)
+        out = run(x)
+        ((out.float() - target) ** 2).mean().backward()
+        return out.detach(), model.network.params.grad.clone(), model.encoding.params.grad.clone()
+
+    y2, dnet2, dtab2 = grads(model.network_with_encoding)
+    y1, dnet1, dtab1 = grads(model)
+    assert torch.equal(y1.view(torch.int16), y2.view(torch.int16))
+    net_scale, tab_scale = float(dnet2.abs().max()), float(dtab2.abs().max())
+    assert torch.allclose(dnet1, dnet2, rtol=2 ** -9, atol=2e-4 * net_scale), float((dnet1 - dnet2).abs().max()) / net_scale
+    # (the two-module route divides dL/d(encoding) by the loss scale in fp16, which at this batch size lies deep in the
+    # subnormal range and keeps few bits; the fused route divides the fp32 sums -- see the test above, where the oracle judges)
+    assert float((dtab1 - dtab2).abs().max()) <= 1e-2 * tab_scale, float((dtab1 - dtab2).abs().max()) / tab_scale
+    assert float(dtab1.abs().sum()) > 0 and torch.isfinite(dtab1).all()
+    # the same model in bf16 has loss scale 1: the same dL/d(encoding) bits reach the scatter on both routes
+    model16 = tcnn.NetworkWithInputEncoding(2, 3, net_config(64, 2), grid, dtype=torch.bfloat16, use_bias=False)
+    with torch.no_grad():
+        model16.encoding.params.copy_(model.encoding.params)
+    model16.train()
+
+    def grads16(run):
+        model16.zero_grad(set_to_none=True)
+        ((run(x).float() - target) ** 2).mean().backward()
+        return model16.encoding.params.grad.clone()
+
+    ta, tb_ = grads16(model16.network_with_encoding), grads16(model16)
+    assert float((ta - tb_).abs().max()) <= 1e-5 * float(ta.abs().max())
+
+
 def test_parameter_free_encodings_through_the_package(tcnn, oracle):
     """test/python/test_encodings.py:377-630 of the reference: spherical harmonics (golden rows), identity, padding, frequency."""
     import json
@@ -691,3 +735,34 @@ def test_image_learning_sample(tcnn, monkeypatch):
     spec.loader.exec_module(sample)
     monkeypatch.setattr(sys, "argv", ["mlp_learning_an_image.py", "--n_steps", "200"])
     assert sample.main() < 1e-3
+
+
+def test_image_learning_sample_on_a_picture_file(tcnn, monkeypatch, tmp_path):
+    """--image: the sample learns a picture read from a file (the reference's sample learns samples/data/images/albert.jpg,
+    samples/mlp_learning_an_image_pytorch.py:128-261; here a small picture written on the spot). The bilinear lookup gives
+    the pixel values at pixel positions and their means half-way between."""
+    import importlib.util
+    import os
+    import sys
+
+    from PIL import Image
+
+    h, w = 48, 64
+    yy, xx = np.mgrid[0:h, 0:w]
+    pic = np.stack([(xx * 255 // (w - 1)), (yy * 255 // (h - 1)), ((xx // 8 + yy // 8) % 2) * 200], axis=2).astype(np.uint8)
+    path_png = str(tmp_path / "picture.png")
+    Image.fromarray(pic, "RGB").save(path_png)
+    path = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "tiny-dpcpp-nn_amd", "samples", "mlp_learning_an_image.py")
+    spec = importlib.util.spec_from_file_location("mlp_learning_an_image_picture", path)
+    sample = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(sample)
+    target = sample.PictureTarget(path_png, DEVICE)
+    at_pixels = torch.tensor([[5 / w, 7 / h], [0.0, 0.0], [(w - 1) / w, (h - 1) / h], [5.5 / w, 7 / h], [1.0, 1.0]], device=DEVICE)
+    got = target(at_pixels).cpu().numpy() * 255
+    np.testing.assert_allclose(got[0], pic[7, 5], atol=1e-3)
+    np.testing.assert_allclose(got[1], pic[0, 0], atol=1e-3)
+    np.testing.assert_allclose(got[2], pic[h - 1, w - 1], atol=1e-3)
+    np.testing.assert_allclose(got[3], (pic[7, 5].astype(np.float64) + pic[7, 6]) / 2, atol=1e-3)
+    np.testing.assert_allclose(got[4], pic[h - 1, w - 1], atol=1e-3)
+    monkeypatch.setattr(sys, "argv", ["mlp_learning_an_image.py", "--n_steps", "300", "--image", path_png])
+    assert sample.main() < 3e-3

@@ -3,11 +3,13 @@
 
 Counterpart of samples/mlp_learning_an_image_pytorch.py of the reference (same model: 2-D HashGrid with 16 levels of 2
 features, log2 hashmap size 15 by default, feeding a 64-wide network with 2 hidden layers; Adam, lr 1e-2; relative L2 loss;
-batches of uniformly random pixel positions). There is no image file to download here: the target is a procedural image
-(smooth colour fields with a few sharp discs), evaluated analytically at the sampled positions. `--ppm out.ppm` writes the
-learned image.
+batches of uniformly random pixel positions). By default the target is a procedural image (smooth colour fields with a few
+sharp discs), evaluated analytically at the sampled positions, so that the sample runs without any file; `--image FILE`
+learns a picture instead (anything Pillow opens, e.g. the reference's samples/data/images/albert.jpg), looked up with
+bilinear filtering as the reference's sample does (:58-91 there). `--ppm out.ppm` writes the learned image.
 
     python tiny-dpcpp-nn_amd/samples/mlp_learning_an_image.py --n_steps 1000
+    python tiny-dpcpp-nn_amd/samples/mlp_learning_an_image.py --image albert.jpg --ppm learned.ppm
 """
 import argparse
 import os
@@ -35,8 +37,34 @@ def target_image(xy):
     return rgb
 
 
+class PictureTarget:
+    """A picture as a function on [0, 1]^2: the value at (x, y) blends the four pixels around (x * width, y * height), pixel
+    (i, j) sitting at the integer position (i, j) and the last row and column repeated beyond the edge."""
+
+    def __init__(self, filename, device):
+        from PIL import Image  # only needed for --image
+
+        rgb = Image.open(filename).convert("RGB")
+        self.width, self.height = rgb.size
+        pixels = torch.frombuffer(bytearray(rgb.tobytes()), dtype=torch.uint8).reshape(self.height * self.width, 3)
+        self.pixels = (pixels.float() / 255.0).to(device)
+
+    def __call__(self, xy):
+        px = xy[:, 0] * self.width
+        py = xy[:, 1] * self.height
+        ix = px.floor().clamp(0, self.width - 1)
+        iy = py.floor().clamp(0, self.height - 1)
+        fx, fy = (px - ix).unsqueeze(1), (py - iy).unsqueeze(1)
+        ix, iy = ix.long(), iy.long()
+        jx, jy = (ix + 1).clamp(max=self.width - 1), (iy + 1).clamp(max=self.height - 1)
+        top = torch.lerp(self.pixels[iy * self.width + ix], self.pixels[iy * self.width + jx], fx)
+        bottom = torch.lerp(self.pixels[jy * self.width + ix], self.pixels[jy * self.width + jx], fx)
+        return torch.lerp(top, bottom, fy)
+
+
 def main():
     ap = argparse.ArgumentParser()
+    ap.add_argument("--image", default=None, help="learn this picture instead of the procedural image")
     ap.add_argument("--n_steps", type=int, default=1000)
     ap.add_argument("--batch_size", type=int, default=2 ** 16)
     ap.add_argument("--log2_hashmap_size", type=int, default=15)
@@ -44,6 +72,7 @@ def main():
     args = ap.parse_args()
 
     device = "cuda"
+    target = PictureTarget(args.image, device) if args.image else target_image
     encoding_config = {"otype": "HashGrid", "n_levels": 16, "n_features_per_level": 2, "log2_hashmap_size": args.log2_hashmap_size,
                        "base_resolution": 16, "per_level_scale": 1.5}
     network_config = {"otype": "FullyFusedMLP", "activation": "ReLU", "output_activation": "None", "n_neurons": 64, "n_hidden_layers": 2}
@@ -53,7 +82,7 @@ def main():
     interval, prev = 10, time.perf_counter()
     for i in range(args.n_steps):
         batch = torch.rand([args.batch_size, 2], device=device)
-        targets = target_image(batch)
+        targets = target(batch)
         output = model(batch).float()
         relative_l2_error = (output - targets) ** 2 / (output.detach() ** 2 + 0.01)
         loss = relative_l2_error.mean()
@@ -75,7 +104,7 @@ def main():
     model.eval()
     with torch.no_grad():
         img = model(xy).float().clamp(0, 1)
-    mse = float(((img - target_image(xy)) ** 2).mean())
+    mse = float(((img - target(xy)) ** 2).mean())
     print(f"mean squared error of the learned {res} x {res} image: {mse:.6f}")
     if args.ppm:
         data = (img.reshape(res, res, 3) * 255).round().to(torch.uint8).cpu().numpy()

@@ -638,7 +638,7 @@ class Bench:
         ach = flops / (tm["ms"] * 1e-3) / 1e12
         roof = {"bound": "mfma", "achieved": ach, "peak": PEAK_MFMA_BF16, "unit": "TFLOP/s", "frac": ach / PEAK_MFMA_BF16, "traffic": None,
                 "kernel": "whole step: mlp_forward_stream_kernel, mlp_layer_backward128_kernel (top layer + loss), "
-                          "mlp_layer_pair_backward128_kernel x (n_hidden / 2), dw_reduce_kernel, mlp_adam_update_kernel",
+                          "mlp_layer_pair_backward128_kernel x (n_hidden / 2), train_reduce_kernel (with Adam)",
                 "kernel_ms": tm["ms"], "algorithmic_flops_per_launch": flops}
         return line("fused-MLP training samples/s (w128, 8 hidden layers, fp16, batch 2^20); % fp16 MFMA peak", "samples/s", "f16",
                     f"training step: w128, 8 hidden layers (9 matmuls), ReLU/linear, fp16, batch 2^{lg}, L2 loss, Adam on fp32 masters (BASELINE config 3, widest)",

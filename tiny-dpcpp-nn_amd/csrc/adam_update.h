@@ -36,19 +36,36 @@ inline AdamArgs make_adam_args(float *master, float *m, float *v, float grad_sca
     return a;
 }
 
-// idx: position in the raw gradient layout, matrix l, [n = out][k = in]; g_raw: the gradient element there.
-template <typename T> __device__ __forceinline__ void adam_update_element(const AdamArgs &a, int idx, float g_raw) {
+// One weight's optimizer state, fetched ahead of the gradient it will be updated with.
+struct AdamElement {
+    int pidx; // position in the packed parameter layout
+    float m, v, w;
+};
+
+// idx: position in the raw gradient layout, matrix l, [n = out][k = in].
+__device__ __forceinline__ AdamElement adam_fetch_element(const AdamArgs &a, int idx) {
     const int W = a.W, per = W * W;
     const int l = idx / per, e = idx % per;
     const int n = e / W, k = e % W;
-    const int pidx = l * per + packed_coord(k, n, W);
+    AdamElement s;
+    s.pidx = l * per + packed_coord(k, n, W);
+    s.m = a.m[s.pidx], s.v = a.v[s.pidx], s.w = a.master[s.pidx];
+    return s;
+}
+
+// g_raw: the gradient element at idx; s: what adam_fetch_element(a, idx) returned.
+template <typename T> __device__ __forceinline__ void adam_apply_element(const AdamArgs &a, int idx, const AdamElement &s, float g_raw) {
+    const int W = a.W, per = W * W;
+    const int l = idx / per, e = idx % per;
+    const int n = e / W, k = e % W;
+    const int pidx = s.pidx;
     const float g = g_raw * a.grad_scale;
-    const float mi = a.m[pidx] + (1.0f - a.beta1) * (g - a.m[pidx]);
-    const float vi = a.beta2 * a.v[pidx] + (1.0f - a.beta2) * g * g;
+    const float mi = s.m + (1.0f - a.beta1) * (g - s.m);
+    const float vi = a.beta2 * s.v + (1.0f - a.beta2) * g * g;
     a.m[pidx] = mi;
     a.v[pidx] = vi;
     const float denom = sqrtf(vi) / a.bc2_sqrt + a.eps;
-    const float p = a.master[pidx] - a.step_size * (mi / denom);
+    const float p = s.w - a.step_size * (mi / denom);
     a.master[pidx] = p;
     const T pt = (T)p;
     if (a.packed_T) static_cast<T *>(a.packed_T)[pidx] = pt;
@@ -57,6 +74,10 @@ template <typename T> __device__ __forceinline__ void adam_update_element(const 
         static_cast<T *>(a.prep_fwd)[(((size_t)l * NI + n / 32) * NK + k / 16) * 512 + (32 * ((k % 16) / 8) + swap23(n % 32)) * 8 + (k % 8)] = pt;
     if (a.prep_bwd) // product index k, contraction index n
         static_cast<T *>(a.prep_bwd)[(((size_t)l * NI + k / 32) * NK + n / 16) * 512 + (32 * ((n % 16) / 8) + swap23(k % 32)) * 8 + (n % 8)] = pt;
+}
+
+template <typename T> __device__ __forceinline__ void adam_update_element(const AdamArgs &a, int idx, float g_raw) {
+    adam_apply_element<T>(a, idx, adam_fetch_element(a, idx), g_raw);
 }
 
 // What follows the main kernel of the fused training step.

@@ -343,7 +343,7 @@ constexpr int kDwSlab = 64; // rows staged in LDS per step
 // Contraction runs over batch rows, which the streaming kernels keep one-per-lane; both operands are
 // therefore transposed through LDS: a slab of rows is stored row-major and read back column-wise.
 // Workgroup (l, c) reduces rows [c*rows_per_chunk, (c+1)*rows_per_chunk) of matrix l into one (or, for
-// W <= 32, four) fp32 partial W x W tiles in the workspace; dw_reduce_kernel sums the partials.
+// W <= 32, four) fp32 partial W x W tiles in the workspace; train_reduce_kernel sums the partials.
 template <typename T, int W>
 __global__ void __launch_bounds__(kDwThreads)
     mlp_dw_partial_kernel(const T *__restrict__ interm_bwd, const T *__restrict__ interm_fwd, float *__restrict__ partials,
@@ -429,50 +429,6 @@ __global__ void __launch_bounds__(kDwThreads)
             const int n = 32 * a + 8 * (r >> 2) + 4 * h + (r & 3);
             const int k = 32 * b + i;
             if (n < W && k < W) out[n * W + k] = acc[tt][r];
-        }
-    }
-}
-
-// Sums the partial tiles in a fixed order. A workgroup of 512 threads owns 64 consecutive elements: each of its 32 groups of
-// 16 lanes (one float4 per lane) adds up every 32nd partial with eight loads in flight, and the group sums are added in
-// group order (one thread per element walking all partials in turn, as this kernel first did, waits for every load: 60 us
-// for 256 partials of a w64 network against 6 us now).
-template <typename T>
-__global__ void __launch_bounds__(512)
-    dw_reduce_kernel(const float *__restrict__ partials, int n_partials, int n_elems, T *__restrict__ dW_T, float *__restrict__ dW_f32) {
-    __shared__ float4 red[32][16];
-    const int c = threadIdx.x & 15, g = threadIdx.x >> 4;
-    const int idx = blockIdx.x * 64 + c * 4; // n_elems is a multiple of 256
-    float4 s[8];
-#pragma unroll
-    for (int u = 0; u < 8; ++u) s[u] = float4{0.f, 0.f, 0.f, 0.f};
-    for (int p0 = g; p0 < n_partials; p0 += 256) {
-#pragma unroll
-        for (int u = 0; u < 8; ++u) {
-            const int p = p0 + 32 * u;
-            if (p < n_partials) {
-                const float4 v = *reinterpret_cast<const float4 *>(partials + (size_t)p * n_elems + idx);
-                s[u].x += v.x; s[u].y += v.y; s[u].z += v.z; s[u].w += v.w;
-            }
-        }
-    }
-    float4 t;
-    t.x = ((s[0].x + s[1].x) + (s[2].x + s[3].x)) + ((s[4].x + s[5].x) + (s[6].x + s[7].x));
-    t.y = ((s[0].y + s[1].y) + (s[2].y + s[3].y)) + ((s[4].y + s[5].y) + (s[6].y + s[7].y));
-    t.z = ((s[0].z + s[1].z) + (s[2].z + s[3].z)) + ((s[4].z + s[5].z) + (s[6].z + s[7].z));
-    t.w = ((s[0].w + s[1].w) + (s[2].w + s[3].w)) + ((s[4].w + s[5].w) + (s[6].w + s[7].w));
-    red[g][c] = t;
-    __syncthreads();
-    if (g == 0) {
-        float4 a = red[0][c];
-#pragma unroll
-        for (int w = 1; w < 32; ++w) {
-            a.x += red[w][c].x; a.y += red[w][c].y; a.z += red[w][c].z; a.w += red[w][c].w;
-        }
-        if (dW_f32) {
-            *reinterpret_cast<float4 *>(dW_f32 + idx) = a;
-        } else {
-            dW_T[idx + 0] = (T)a.x; dW_T[idx + 1] = (T)a.y; dW_T[idx + 2] = (T)a.z; dW_T[idx + 3] = (T)a.w;
         }
     }
 }
@@ -698,36 +654,46 @@ static int launch_dw(const tnn_mlp_desc *d, const void *interm_bwd, const void *
     int rc = check_launch("mlp_dw_partial_kernel");
     if (rc) return rc;
     const int n_elems = n_mats * W * W;
-    TNN_LAUNCH((dw_reduce_kernel<T>), dim3(n_elems / 64), dim3(512), 0, s, partials,
-                       (int)(p.n_chunks * p.partials_per_chunk), n_elems, dW_is_fp32 ? (T *)nullptr : (T *)dW,
-                       dW_is_fp32 ? (float *)dW : (float *)nullptr);
-    return check_launch("dw_reduce_kernel");
+    TNN_LAUNCH((train_reduce_kernel<T, false>), dim3(n_elems / 64), dim3(512), 0, s, partials, (const float *)nullptr,
+               (int)(p.n_chunks * p.partials_per_chunk), n_elems, dW_is_fp32 ? (T *)nullptr : (T *)dW,
+               dW_is_fp32 ? (float *)dW : (float *)nullptr, (float *)nullptr, AdamArgs{});
+    return check_launch("train_reduce_kernel");
 }
 
 // Width 128: one launch per layer that forms delta_{l-1} and dW_l together (mlp_backward128.inc), then the reduction.
-// With `targets` the top layer's launch forms dL/dy itself from the network's output (the last matrix of interm_fwd) and adds
-// the loss values into *loss_sum (zeroed by the caller); dLdy is then not read.
+// With `targets` the top layer's launch forms dL/dy itself from the network's output (the last matrix of interm_fwd) and leaves
+// the loss values as one sum per workgroup, which the reduction adds into *loss_sum; dLdy is then not read, and `tail` may ask
+// for Adam on the reduced gradients inside the reduction (dW may then be null).
 template <typename T>
 static int launch_backward128(const tnn_mlp_desc *d, const void *wprep_bwd, const void *dLdy, const void *interm_fwd, void *deltas,
                               bool keep_top_delta, void *dW, int dW_is_fp32, void *dLdx, size_t M, float *partials, hipStream_t s,
-                              const float *targets = nullptr, float loss_scale = 0.0f, float *loss_sum = nullptr, const void *x0 = nullptr) {
+                              const float *targets = nullptr, float loss_scale = 0.0f, float *loss_sum = nullptr, const void *x0 = nullptr,
+                              const void *wprep_fwd = nullptr, // (with targets): the network's output is not in interm_fwd, the top launch forms it
+                              const TrainTail &tail = TrainTail{}) {
     typedef typename Storage<T>::vec8 vec8;
     constexpr int W = 128;
     const int n_mats = d->n_hidden_layers + 1;
     const DwPlan p = dw_plan(d, M);
     const size_t mat = M * W, per_mat = (size_t)4 * 8 * 64;
-    auto k_top = targets ? mlp_layer_backward128_kernel<T, 2> : mlp_layer_backward128_kernel<T, 1>;
+    const bool reform = targets && wprep_fwd;
+    auto k_top = reform ? mlp_layer_backward128_kernel<T, 3> : (targets ? mlp_layer_backward128_kernel<T, 2> : mlp_layer_backward128_kernel<T, 1>);
     auto k_mid = mlp_layer_backward128_kernel<T, 0>;
     auto k_pair = mlp_layer_pair_backward128_kernel<T>;
     const float inv_n = 1.0f / (float)(M * W);
-    for (auto k : {k_top, k_mid})
-        if (hipFuncSetAttribute(reinterpret_cast<const void *>(k), hipFuncAttributeMaxDynamicSharedMemorySize, (int)LayerBwd128::lds_bytes) != hipSuccess)
-            return fail(TNN_ERR_HIP, "cannot reserve %zu bytes of LDS", LayerBwd128::lds_bytes);
+    const size_t top_lds = reform ? LayerBwd128::pair_lds_bytes : LayerBwd128::lds_bytes;
+    if (hipFuncSetAttribute(reinterpret_cast<const void *>(k_top), hipFuncAttributeMaxDynamicSharedMemorySize, (int)top_lds) != hipSuccess)
+        return fail(TNN_ERR_HIP, "cannot reserve %zu bytes of LDS", top_lds);
+    if (hipFuncSetAttribute(reinterpret_cast<const void *>(k_mid), hipFuncAttributeMaxDynamicSharedMemorySize, (int)LayerBwd128::lds_bytes) != hipSuccess)
+        return fail(TNN_ERR_HIP, "cannot reserve %zu bytes of LDS", LayerBwd128::lds_bytes);
     if (hipFuncSetAttribute(reinterpret_cast<const void *>(k_pair), hipFuncAttributeMaxDynamicSharedMemorySize, (int)LayerBwd128::pair_lds_bytes) != hipSuccess)
         return fail(TNN_ERR_HIP, "cannot reserve %zu bytes of LDS", LayerBwd128::pair_lds_bytes);
     const T *fwd = static_cast<const T *>(interm_fwd);
     const T *input0 = x0 ? static_cast<const T *>(x0) : fwd; // the first matrix's input: the caller's x, or its copy in front of the activations
     T *dl = static_cast<T *>(deltas);
+    // from the loss nobody keeps the top layer's deltas: the workgroups' loss sums lie in that matrix's place
+    float *loss_partials = (targets && loss_sum && !keep_top_delta && mat * sizeof(T) >= (size_t)p.n_chunks * sizeof(float))
+                               ? reinterpret_cast<float *>(dl + (size_t)(n_mats - 1) * mat) : (float *)nullptr;
+    if (targets && loss_sum && !loss_partials) return fail(TNN_ERR_INVALID_ARGUMENT, "no room for the loss sums of %lld workgroups", p.n_chunks);
     const vec8 *wb = static_cast<const vec8 *>(wprep_bwd);
     // the top layer by itself (it turns dL/dy or the loss into deltas first), then the layers below it two per launch, and
     // the first matrix by itself when their number is odd
@@ -748,30 +714,48 @@ static int launch_backward128(const tnn_mlp_desc *d, const void *wprep_bwd, cons
         const T *delta_in = top ? static_cast<const T *>(dLdy) : dl + (size_t)l * mat;
         T *delta_out = l > 0 ? dl + (size_t)(l - 1) * mat : static_cast<T *>(dLdx);
         const int gate = l > 0 ? d->activation : TNN_ACT_NONE;
-        TNN_LAUNCH((top ? k_top : k_mid), dim3((unsigned)p.n_chunks), dim3(kLayerBwdThreads), LayerBwd128::lds_bytes, s, wb + (size_t)l * per_mat,
-                   delta_in, l > 0 ? fwd + (size_t)l * mat : input0, fwd + (size_t)n_mats * mat, (top && keep_top_delta) ? dl + (size_t)l * mat : (T *)nullptr,
-                   delta_out, partials, n_mats, l, gate, d->output_activation, (long long)M, p.rows_per_chunk, targets, loss_scale, inv_n, loss_sum);
+        TNN_LAUNCH((top ? k_top : k_mid), dim3((unsigned)p.n_chunks), dim3(kLayerBwdThreads), top ? top_lds : LayerBwd128::lds_bytes, s,
+                   wb + (size_t)l * per_mat, delta_in, l > 0 ? fwd + (size_t)l * mat : input0, fwd + (size_t)n_mats * mat,
+                   (top && keep_top_delta) ? dl + (size_t)l * mat : (T *)nullptr, delta_out, partials, n_mats, l, gate, d->output_activation, (long long)M,
+                   p.rows_per_chunk, targets, loss_scale, inv_n, loss_partials,
+                   (top && reform) ? static_cast<const vec8 *>(wprep_fwd) + (size_t)l * per_mat : (const vec8 *)nullptr);
         const int rc = check_launch("mlp_layer_backward128_kernel");
         if (rc) return rc;
         l -= 1;
     }
+    if (tail.main_done && hipEventRecord(tail.main_done, s) != hipSuccess) return fail(TNN_ERR_HIP, "hipEventRecord failed");
     const int n_elems = n_mats * W * W;
-    TNN_LAUNCH((dw_reduce_kernel<T>), dim3(n_elems / 64), dim3(512), 0, s, partials, (int)(p.n_chunks * p.partials_per_chunk), n_elems,
-               dW_is_fp32 ? (T *)nullptr : (T *)dW, dW_is_fp32 ? (float *)dW : (float *)nullptr);
-    return check_launch("dw_reduce_kernel");
+    T *dW_T = (dW && !dW_is_fp32) ? (T *)dW : (T *)nullptr;
+    float *dW_f32 = (dW && dW_is_fp32) ? (float *)dW : (float *)nullptr;
+    if (tail.use_adam)
+        TNN_LAUNCH((train_reduce_kernel<T, true>), dim3(n_elems / 64), dim3(512), 0, s, partials, loss_partials, (int)p.n_chunks, n_elems, dW_T, dW_f32,
+                   loss_partials ? loss_sum : (float *)nullptr, tail.adam);
+    else
+        TNN_LAUNCH((train_reduce_kernel<T, false>), dim3(n_elems / 64), dim3(512), 0, s, partials, loss_partials, (int)p.n_chunks, n_elems, dW_T, dW_f32,
+                   loss_partials ? loss_sum : (float *)nullptr, tail.adam);
+    return check_launch("train_reduce_kernel");
 }
 
 // For tnn_mlp_train_step_l2 on width 128. The forward pass with stored activations that does not copy the input in front of
 // them where its kernel can leave that out (2^20 rows: 268 MB less to write), ...
-int forward128_for_training(const tnn_mlp_desc *desc, const void *wprep, const void *x, void *interm_fwd, size_t M, hipStream_t s) {
-    if (desc->dtype == TNN_BF16) return launch_forward<bf16_t, 128, true>(desc, wprep, x, interm_fwd, M, s, false);
-    return launch_forward<fp16_t, 128, true>(desc, wprep, x, interm_fwd, M, s, false);
+// without_output: the last layer is left out (the backward pass's top launch forms the network's output again from the last
+// hidden layer, which lies where it always does); needs at least two hidden layers.
+int forward128_for_training(const tnn_mlp_desc *desc, const void *wprep, const void *x, void *interm_fwd, size_t M, hipStream_t s, bool without_output) {
+    tnn_mlp_desc d = *desc;
+    if (without_output) {
+        d.n_hidden_layers -= 1;
+        d.output_activation = d.activation; // the last matrix that runs is a hidden layer's
+    }
+    if (desc->dtype == TNN_BF16) return launch_forward<bf16_t, 128, true>(&d, wprep, x, interm_fwd, M, s, false);
+    return launch_forward<fp16_t, 128, true>(&d, wprep, x, interm_fwd, M, s, false);
 }
 
 // ... and loss and backward pass over those activations, the loss folded into the top layer's launch and the first matrix's
 // input read from `x`. Workspace as tnn_mlp_backward's.
+// wprep_fwd_if_no_output: the operand-order weights of the forward pass when interm_fwd holds no network output (see above), else null.
 int backward128_from_loss(const tnn_mlp_desc *desc, const void *wprep_bwd, const void *x, const void *interm_fwd, const float *targets, float loss_scale,
-                          float *loss_sum, void *dW, int dW_is_fp32, void *dLdx, size_t M, void *workspace, size_t workspace_bytes, hipStream_t s) {
+                          float *loss_sum, void *dW, int dW_is_fp32, void *dLdx, size_t M, void *workspace, size_t workspace_bytes, hipStream_t s,
+                          const void *wprep_fwd_if_no_output, const TrainTail &tail) {
     const DwPlan p = dw_plan(desc, M);
     const size_t partial_rounded = (p.partial_bytes + 255) & ~(size_t)255;
     const size_t need = partial_rounded + p.delta_bytes + 512;
@@ -781,9 +765,9 @@ int backward128_from_loss(const tnn_mlp_desc *desc, const void *wprep_bwd, const
     void *deltas = reinterpret_cast<void *>(base + partial_rounded);
     if (desc->dtype == TNN_BF16)
         return launch_backward128<bf16_t>(desc, wprep_bwd, nullptr, interm_fwd, deltas, false, dW, dW_is_fp32, dLdx, M, partials, s, targets, loss_scale,
-                                          loss_sum, x);
+                                          loss_sum, x, wprep_fwd_if_no_output, tail);
     return launch_backward128<fp16_t>(desc, wprep_bwd, nullptr, interm_fwd, deltas, false, dW, dW_is_fp32, dLdx, M, partials, s, targets, loss_scale,
-                                      loss_sum, x);
+                                      loss_sum, x, wprep_fwd_if_no_output, tail);
 }
 
 #define TNN_DISPATCH_TW(desc, CALL)                                                          \

@@ -38,9 +38,10 @@ int fused_train_step(const tnn_mlp_desc *d, const void *wf, const void *wb, cons
                      hipStream_t s);
 size_t fused_train_workspace_bytes(const tnn_mlp_desc *d, size_t M);
 // mlp.hip
-int forward128_for_training(const tnn_mlp_desc *desc, const void *wprep, const void *x, void *interm_fwd, size_t M, hipStream_t s);
+int forward128_for_training(const tnn_mlp_desc *desc, const void *wprep, const void *x, void *interm_fwd, size_t M, hipStream_t s, bool without_output);
 int backward128_from_loss(const tnn_mlp_desc *desc, const void *wprep_bwd, const void *x, const void *interm_fwd, const float *targets, float loss_scale,
-                          float *loss_sum, void *dW, int dW_is_fp32, void *dLdx, size_t M, void *workspace, size_t workspace_bytes, hipStream_t s);
+                          float *loss_sum, void *dW, int dW_is_fp32, void *dLdx, size_t M, void *workspace, size_t workspace_bytes, hipStream_t s,
+                          const void *wprep_fwd_if_no_output, const TrainTail &tail);
 
 } // namespace tnn
 
@@ -55,6 +56,10 @@ TNN_API size_t tnn_mlp_train_step_workspace_bytes(const tnn_mlp_desc *desc, size
     return align256((size_t)(desc->n_hidden_layers + 2) * mat) + align256(mat) + align256(tnn_mlp_backward_workspace_bytes(desc, M)) +
            align256(unfused_dw_bytes(desc)) + 512;
 }
+
+static int unfused_train_step(const tnn_mlp_desc *desc, const void *d_prepared_fwd, const void *d_prepared_bwd, const void *d_x, const float *d_targets,
+                              float loss_scale, void *d_y, float *d_loss_sum, void *d_dW, int dW_is_fp32, void *d_dLdx, size_t M, void *d_workspace,
+                              const TrainTail &tail, tnn_stream_t stream);
 
 TNN_API int tnn_mlp_train_step_l2(const tnn_mlp_desc *desc, const void *d_prepared_fwd, const void *d_prepared_bwd,
                                   const void *d_x, const float *d_targets, float loss_scale, void *d_y, float *d_loss_sum,
@@ -73,7 +78,17 @@ TNN_API int tnn_mlp_train_step_l2(const tnn_mlp_desc *desc, const void *d_prepar
     rc = fused_train_step(desc, d_prepared_fwd, d_prepared_bwd, d_x, d_targets, loss_scale, d_y, d_loss_sum, d_dW, dW_is_fp32, d_dLdx, M,
                           d_workspace, workspace_bytes, TrainTail{}, s);
     if (rc != TNN_ERR_UNSUPPORTED) return rc;
-    // wider / deeper networks: forward, loss and backward as separate kernels over workspace matrices
+    return unfused_train_step(desc, d_prepared_fwd, d_prepared_bwd, d_x, d_targets, loss_scale, d_y, d_loss_sum, d_dW, dW_is_fp32, d_dLdx, M, d_workspace,
+                              TrainTail{}, stream);
+}
+
+// Wider / deeper networks than the fused kernel takes: forward, loss and backward as separate kernels over workspace matrices
+// (arguments checked by the caller, the workspace at least tnn_mlp_train_step_workspace_bytes). `tail` with Adam: width 128 only.
+static int unfused_train_step(const tnn_mlp_desc *desc, const void *d_prepared_fwd, const void *d_prepared_bwd, const void *d_x, const float *d_targets,
+                              float loss_scale, void *d_y, float *d_loss_sum, void *d_dW, int dW_is_fp32, void *d_dLdx, size_t M, void *d_workspace,
+                              const TrainTail &tail, tnn_stream_t stream) {
+    int rc;
+    hipStream_t s = as_stream(stream);
     const int W = desc->width, n_mats = desc->n_hidden_layers + 1;
     const size_t mat = M * W * 2;
     uintptr_t base = align256(reinterpret_cast<uintptr_t>(d_workspace));
@@ -84,14 +99,18 @@ TNN_API int tnn_mlp_train_step_l2(const tnn_mlp_desc *desc, const void *d_prepar
     void *bwd_ws = reinterpret_cast<void *>(base);
     const size_t bwd_ws_bytes = align256(tnn_mlp_backward_workspace_bytes(desc, M));
 
-    if ((rc = (W == 128 ? forward128_for_training(desc, d_prepared_fwd, d_x, interm_fwd, M, s) : tnn_mlp_forward(desc, d_prepared_fwd, d_x, interm_fwd, M, stream)))) return rc;
+    // width 128 when nobody asks for the network's output: the forward pass ends at the last hidden layer and the backward
+    // pass's first launch forms the output again on chip (one matrix less to write and to read)
+    const bool no_output = W == 128 && !d_y && desc->n_hidden_layers >= 2;
+    if ((rc = (W == 128 ? forward128_for_training(desc, d_prepared_fwd, d_x, interm_fwd, M, s, no_output) : tnn_mlp_forward(desc, d_prepared_fwd, d_x, interm_fwd, M, stream)))) return rc;
     const void *y = static_cast<const char *>(interm_fwd) + (size_t)n_mats * mat;
     if (d_y && hipMemcpyAsync(d_y, y, mat, hipMemcpyDeviceToDevice, s) != hipSuccess) return fail(TNN_ERR_HIP, "copy of the network output failed");
     const size_t n = M * W;
-    if (d_loss_sum) TNN_LAUNCH(zero_scalar_kernel, dim3(1), dim3(1), 0, s, d_loss_sum);
-    // width 128: the loss is part of the backward pass's first launch (dL/dy is never written)
+    // width 128: the loss is part of the backward pass's first launch (dL/dy is never written), its sum and, when asked for,
+    // Adam are part of the reduction that ends the pass
     if (W == 128) return backward128_from_loss(desc, d_prepared_bwd, d_x, interm_fwd, d_targets, loss_scale, d_loss_sum, d_dW, dW_is_fp32, d_dLdx, M, bwd_ws,
-                                               bwd_ws_bytes, s);
+                                               bwd_ws_bytes, s, no_output ? d_prepared_fwd : nullptr, tail);
+    if (d_loss_sum) TNN_LAUNCH(zero_scalar_kernel, dim3(1), dim3(1), 0, s, d_loss_sum);
     size_t blocks = (n + 256 * 8 - 1) / (256 * 8);
     if (blocks > 2048) blocks = 2048;
     const float inv_n = 1.0f / (float)n;
@@ -129,7 +148,11 @@ TNN_API int tnn_mlp_train_step_l2_adam(const tnn_mlp_desc *desc, void *d_prepare
     rc = fused_train_step(desc, d_prepared_fwd, d_prepared_bwd, d_x, d_targets, loss_scale, d_y, d_loss_sum, nullptr, 1, d_dLdx, M,
                           d_workspace, workspace_bytes, tail, s);
     if (rc != TNN_ERR_UNSUPPORTED) return rc;
-    // no fused kernel for this shape: the separate step, then the separate update, over gradients kept in the workspace
+    // width 128: separate kernels, the update inside the reduction that ends the backward pass (no gradient tensor)
+    if (desc->width == 128)
+        return unfused_train_step(desc, d_prepared_fwd, d_prepared_bwd, d_x, d_targets, loss_scale, d_y, d_loss_sum, nullptr, 1, d_dLdx, M, d_workspace, tail,
+                                  stream);
+    // other shapes without a fused kernel: the separate step, then the separate update, over gradients kept in the workspace
     const uintptr_t end = reinterpret_cast<uintptr_t>(d_workspace) + workspace_bytes;
     float *dW = reinterpret_cast<float *>((end - unfused_dw_bytes(desc)) & ~(uintptr_t)255);
     // (the step lays its matrices out from the front of the workspace and stays clear of this tail)

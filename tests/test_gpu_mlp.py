@@ -495,6 +495,63 @@ def test_baseline_config_3_full_size(tnn, oracle, W, n_hidden):
     diff, bar = np.abs(dXh - rdX), 5e-4 * np.abs(rdX).max() + 5e-3 * np.abs(rdX)
     assert (diff <= bar).all(axis=1).mean() >= 0.98
     assert np.linalg.norm((dXh - rdX).ravel()) <= 2e-2 * np.linalg.norm(rdX.ravel())
+    # The same gradients at the bar of every other end-to-end check, with the masks taken out of the comparison: the oracle's
+    # backward pass over the activations the GPU's forward pass stores (the step's own, bit for bit: same kernel, and its
+    # output is checked to be theirs), so both sides gate with the same ReLU masks and differ only by the rounding of the deltas.
+    interm_t = tnn.forward(desc, pf, xs)
+    assert torch.equal(ys_, interm_t[-1])
+    interm_g = tnn.host(interm_t)
+    _, grads_g = oracle.l2_loss(dtype, interm_g[-1], ts.cpu().numpy(), 4096.0)
+    _, rdW_g, rdX_g = oracle.mlp_backward_T(dtype, W, n_mats, "relu", "none", w, interm_g, grads_g, round_dw=False)
+    assert_propagated(dXh, rdX_g, dtype, "dL/dx of the sub-batch over the GPU's activations", scale=float(np.abs(rdX_g).max()))
+    assert_propagated(dWs.cpu().numpy(), rdW_g, dtype, "dW of the sub-batch over the GPU's activations", scale=float(np.abs(rdW_g).max()))
+
+
+@pytest.mark.parametrize("dtype,n_hidden,act,out_act,M", [(FP16, 8, "relu", "none", (1 << 16) + 8 * 37), (BF16, 3, "relu", "sigmoid", 1 << 16),
+                                                          (FP16, 2, "sigmoid", "none", (1 << 17) + 8), (BF16, 5, "relu", "relu", (1 << 16) + 2048)])
+def test_width_128_step_without_stored_output(tnn, oracle, dtype, n_hidden, act, out_act, M):
+    """A width-128 training step that is not asked for the network's output ends its forward pass at the last hidden layer;
+    the top launch of its backward pass forms the output again with the forward pass's arithmetic. Everything it returns
+    must be what the step with the output stored returns: dL/dx bit for bit, the weight gradients bit for bit as well (same
+    partial sums over the same values), the loss to the rounding of its sum. Odd and even numbers of matrices (the bottom
+    layer alone or in a pair), ragged last rounds, every output activation; the batch sizes are those of the streaming
+    forward kernel (the small ones are in test_train_step_single_call)."""
+    import torch
+    W, n_mats = 128, n_hidden + 1
+    w = oracle.round(xavier(W, n_mats, 11), dtype)
+    desc = tnn.mlp_desc(dtype, W, n_hidden, act, out_act)
+    _, pf, pb = tnn.prepare(desc, w)
+    gen = torch.Generator(device=tnn.dev).manual_seed(21)
+    x = (torch.rand((M, W), device=tnn.dev, generator=gen) * 2 - 1).to(torch.float16 if dtype == FP16 else torch.bfloat16)
+    targets = torch.rand((M, W), device=tnn.dev, generator=gen)
+    ls = 128.0 * M / 1024
+    y, loss, dW, dX = tnn.train_step_l2(desc, pf, pb, x, targets, ls, want_y=True, want_dx=True, dw_fp32=True)
+    y2, loss2, dW2, dX2 = tnn.train_step_l2(desc, pf, pb, x, targets, ls, want_y=False, want_dx=True, dw_fp32=True)
+    assert y2 is None
+    assert torch.equal(dX2.view(torch.int16), dX.view(torch.int16))
+    assert torch.equal(dW2.view(torch.int32), dW.view(torch.int32))
+    assert abs(float(loss2) - float(loss)) <= 1e-6 * abs(float(loss))
+    # the step with the optimizer inside takes the same route: one step from zero moments against the oracle's Adam on dW
+    from gpu_harness import ptr
+    from tiny_dpcpp_nn import _lib
+    master = tnn.pack(FP32, W, n_mats, torch.from_numpy(w.reshape(-1)).to(tnn.dev))
+    dWp = torch.empty(n_mats * W * W, dtype=torch.float32, device=tnn.dev)
+    _lib.check(tnn.lib.tnn_pack_and_transpose(2, W, n_mats, ptr(dW), ptr(dWp), tnn.stream()))
+    rp, rm, rv = oracle.adam_step(tnn.host(master), np.zeros(master.numel(), np.float32), np.zeros(master.numel(), np.float32),
+                                  tnn.host(dWp) / np.float32(ls), 1, 1e-2, 0.9, 0.999, 1e-8)
+    pf2, pb2 = tnn.prepare_packed(desc, master, src_is_fp32=True)
+    m, v = torch.zeros_like(master), torch.zeros_like(master)
+    ws_bytes = tnn.lib.tnn_mlp_train_step_workspace_bytes(ctypes.byref(desc), M)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=tnn.dev)
+    loss3 = torch.full((1,), float("nan"), device=tnn.dev)
+    _lib.check(tnn.lib.tnn_mlp_train_step_l2_adam(ctypes.byref(desc), ptr(pf2), ptr(pb2), ptr(x), ptr(targets), ls, None, ptr(loss3), ptr(master),
+                                                  ptr(m), ptr(v), 1, 1e-2, 0.9, 0.999, 1e-8, None, None, M, ptr(ws), ws_bytes, None, tnn.stream()))
+    tnn.sync()
+    assert abs(float(loss3) - float(loss)) <= 1e-6 * abs(float(loss))
+    assert np.allclose(tnn.host(m), rm, rtol=1e-5, atol=1e-12) and np.allclose(tnn.host(v), rv, rtol=1e-5, atol=1e-20)
+    assert np.allclose(tnn.host(master), rp, rtol=1e-6, atol=2e-6)
+    wf_ref, wb_ref = tnn.prepare_packed(desc, master, src_is_fp32=True)
+    assert torch.equal(pf2.view(torch.int16), wf_ref.view(torch.int16)) and torch.equal(pb2.view(torch.int16), wb_ref.view(torch.int16))
 
 
 @pytest.mark.parametrize("dtype,W,n_hidden,log2_m", [(FP16, 16, 2, 19), (FP16, 16, 4, 19), (BF16, 32, 2, 19), (BF16, 64, 4, 18), (FP16, 64, 2, 17)])

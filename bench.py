@@ -49,6 +49,8 @@ MEASURED_TRAFFIC_BYTES = {
     ("grid_mlp_ordered", 21): (3915783.4 * 2.0 + 264728.9) * 1024,
     ("grid_train", 18): (108943.2 * 2.0 + 236762.7) * 1024,  # the scatter kernel; an atomic request counts as a 32-byte write
     ("grid_train_ordered", 18): (248862.1 * 2.0 + 126583.5) * 1024,
+    # the whole width-128 step: forward, top launch, four pair launches, reduction with Adam
+    ("train_w128", 20): ((138126.3 + 403751.0 + 4 * 393607.4 + 77222.7) * 2.0 + (2098630.8 + 283206.9 + 4 * 229381.6 + 8674.3)) * 1024,
 }
 
 
@@ -636,7 +638,8 @@ class Bench:
         flops = 3 * 2 * M * W * W * n_mats
         lg = int(np.log2(M))
         ach = flops / (tm["ms"] * 1e-3) / 1e12
-        roof = {"bound": "mfma", "achieved": ach, "peak": PEAK_MFMA_BF16, "unit": "TFLOP/s", "frac": ach / PEAK_MFMA_BF16, "traffic": None,
+        roof = {"bound": "mfma", "achieved": ach, "peak": PEAK_MFMA_BF16, "unit": "TFLOP/s", "frac": ach / PEAK_MFMA_BF16,
+                "traffic": MEASURED_TRAFFIC_BYTES.get(("train_w128", lg)),
                 "kernel": "whole step: mlp_forward_stream_kernel, mlp_layer_backward128_kernel (top layer + loss), "
                           "mlp_layer_pair_backward128_kernel x (n_hidden / 2), train_reduce_kernel (with Adam)",
                 "kernel_ms": tm["ms"], "algorithmic_flops_per_launch": flops}

@@ -467,6 +467,50 @@ def test_fused_training_route_at_a_batch_that_is_visited_in_cell_order(tcnn):
     assert float((ta - tb_).abs().max()) <= 1e-5 * float(ta.abs().max())
 
 
+def test_backward_takes_over_the_forward_pass_cell_order_only_when_it_is_that_batch_s(tcnn):
+    """The fused forward pass of a training step orders a large batch by cell and the backward pass uses that order again
+    instead of forming it a second time; the native module keeps one order, the last one formed. Two forward passes on
+    different batches followed by the backward pass of the FIRST must therefore order the first batch again (its order is no
+    longer the one kept); the backward pass of the second then finds its own order gone as well. Gradients of both must be
+    what each batch gives on its own."""
+    torch.manual_seed(31)
+    grid = {"otype": "HashGrid", "n_levels": 16, "n_features_per_level": 2, "log2_hashmap_size": 19, "base_resolution": 16, "per_level_scale": 1.5}
+    model = tcnn.NetworkWithInputEncoding(2, 3, net_config(64, 2), grid, dtype=torch.bfloat16, use_bias=False)
+    with torch.no_grad():
+        model.encoding.params.copy_(torch.rand_like(model.encoding.params) * 2 - 1)
+    model.train()
+    batch = 1 << 17
+    xa, xb = torch.rand((batch, 2), device=DEVICE), torch.rand((batch, 2), device=DEVICE)
+    ta, tb = torch.rand((batch, 3), device=DEVICE), torch.rand((batch, 3), device=DEVICE)
+
+    def alone(x, t):
+        model.zero_grad(set_to_none=True)
+        ((model(x).float() - t) ** 2).mean().backward()  # forward orders, backward takes the order over
+        return model.network.params.grad.clone(), model.encoding.params.grad.clone()
+
+    na, ea = alone(xa, ta)
+    nb, eb = alone(xb, tb)
+    model.zero_grad(set_to_none=True)
+    la = ((model(xa).float() - ta) ** 2).mean()
+    lb = ((model(xb).float() - tb) ** 2).mean()  # the order kept is now xb's
+    la.backward()  # must not scatter xa's gradients over xb's order
+    n1, e1 = model.network.params.grad.clone(), model.encoding.params.grad.clone()
+    model.zero_grad(set_to_none=True)
+    lb.backward()  # and the order kept is xa's again
+    n2, e2 = model.network.params.grad.clone(), model.encoding.params.grad.clone()
+    for got, want in ((n1, na), (e1, ea), (n2, nb), (e2, eb)):
+        scale = float(want.abs().max())
+        assert scale > 0
+        assert float((got - want).abs().max()) <= 1e-4 * scale, float((got - want).abs().max()) / scale
+    # a batch written to in place after its forward pass: autograd refuses the backward pass (which is what lets it reuse the order)
+    model.zero_grad(set_to_none=True)
+    xc = xa.clone()
+    lc = ((model(xc).float() - ta) ** 2).mean()
+    xc.mul_(0.5)
+    with pytest.raises(RuntimeError, match="modified by an inplace operation"):
+        lc.backward()
+
+
 def test_parameter_free_encodings_through_the_package(tcnn, oracle):
     """test/python/test_encodings.py:377-630 of the reference: spherical harmonics (golden rows), identity, padding, frequency."""
     import json
@@ -668,7 +712,7 @@ def test_modules_follow_the_callers_stream(tcnn):
 
 
 def test_large_batches_take_the_cell_order_route(tcnn):
-    """From 2^19 rows on the grid encoding (alone, and fused with the network) orders the batch by cell first. Row for row the
+    """From 2^19 rows on the grid encoding alone, and from 2^18 on fused with the network, orders the batch by cell first. Row for row the
     result equals what the same rows give in batches below the threshold."""
     n = (1 << 19) + 40
     cfg = {"otype": "HashGrid", "n_levels": 16, "n_features_per_level": 2, "log2_hashmap_size": 17, "base_resolution": 16, "per_level_scale": 1.447}

@@ -55,9 +55,9 @@ class PybindingModule {
     }
     /// Network modules: whether inference on `encoding`'s output can run as one kernel, and that inference.
     bool can_fuse_encoding(const PybindingModule &encoding) const { return m_module->can_fuse_encoding(*encoding.m_module); }
-    torch::Tensor inference_with_encoding(const PybindingModule &encoding, torch::Tensor positions) {
+    torch::Tensor inference_with_encoding(const PybindingModule &encoding, torch::Tensor positions, bool a_backward_pass_follows) {
         CHECK_INPUT(positions);
-        return m_module->inference_with_encoding(*encoding.m_module, positions);
+        return m_module->inference_with_encoding(*encoding.m_module, positions, a_backward_pass_follows);
     }
     /// Network modules, training without stored activations: inference() is the forward pass, these are the backward passes.
     bool can_recompute_backward() const { return m_module->can_recompute_backward(); }
@@ -68,10 +68,10 @@ class PybindingModule {
     }
     bool can_train_with_encoding(const PybindingModule &encoding) const { return m_module->can_train_with_encoding(*encoding.m_module); }
     std::tuple<torch::Tensor, torch::Tensor> bwd_with_encoding(const PybindingModule &encoding, torch::Tensor positions, torch::Tensor grad_output,
-                                                               bool pack_gradient) {
+                                                               bool pack_gradient, bool positions_unchanged_since_forward) {
         CHECK_INPUT(positions);
         CHECK_INPUT(grad_output);
-        return m_module->backward_with_encoding(*encoding.m_module, positions, grad_output, pack_gradient);
+        return m_module->backward_with_encoding(*encoding.m_module, positions, grad_output, pack_gradient, positions_unchanged_since_forward);
     }
     torch::Tensor initial_params() { return m_module->initialize_params(); }
     torch::Tensor initial_params(torch::Tensor &tensor) { return m_module->initialize_params(tensor); }
@@ -129,11 +129,13 @@ PYBIND11_MODULE(tiny_dpcpp_nn_pybind_module, m) {
         .def("fwd", &PybindingModule::fwd)
         .def("inference", &PybindingModule::inference)
         .def("can_fuse_encoding", &PybindingModule::can_fuse_encoding)
-        .def("inference_with_encoding", &PybindingModule::inference_with_encoding)
+        .def("inference_with_encoding", &PybindingModule::inference_with_encoding, py::arg("encoding"), py::arg("positions"),
+             py::arg("a_backward_pass_follows") = false)
         .def("can_recompute_backward", &PybindingModule::can_recompute_backward)
         .def("bwd_recompute", &PybindingModule::bwd_recompute)
         .def("can_train_with_encoding", &PybindingModule::can_train_with_encoding)
-        .def("bwd_with_encoding", &PybindingModule::bwd_with_encoding)
+        .def("bwd_with_encoding", &PybindingModule::bwd_with_encoding, py::arg("encoding"), py::arg("positions"), py::arg("grad_output"),
+             py::arg("pack_gradient"), py::arg("positions_unchanged_since_forward") = false)
         .def("bwd_no_encoding_grad", &PybindingModule::bwd_no_encoding_grad)
         .def("bwd_with_encoding_grad", &PybindingModule::bwd_with_encoding_grad)
         .def("initial_params", py::overload_cast<>(&PybindingModule::initial_params))

@@ -56,7 +56,7 @@ class Module {
     /// No counterpart in the reference (NetworkWithInputEncoding runs the two modules in turn,
     /// dpcpp_bindings/tiny_dpcpp_nn/modules.py:357-421); the values are those of the two calls.
     virtual bool can_fuse_encoding(const Module &) const { return false; }
-    virtual torch::Tensor inference_with_encoding(const Module &, const torch::Tensor &) {
+    virtual torch::Tensor inference_with_encoding(const Module &, const torch::Tensor &, bool = false) {
         throw std::runtime_error("inference_with_encoding: not a network module");
     }
 
@@ -71,7 +71,7 @@ class Module {
     /// The same behind a grid encoding: inference_with_encoding() is the forward pass, backward_with_encoding returns the
     /// network's weight gradients (packed on request) and the gradient of the encoding's table.
     virtual bool can_train_with_encoding(const Module &) const { return false; }
-    virtual std::tuple<torch::Tensor, torch::Tensor> backward_with_encoding(const Module &, const torch::Tensor &, const torch::Tensor &, bool) {
+    virtual std::tuple<torch::Tensor, torch::Tensor> backward_with_encoding(const Module &, const torch::Tensor &, const torch::Tensor &, bool, bool = false) {
         throw std::runtime_error("backward_with_encoding: not a network module");
     }
 
@@ -321,7 +321,9 @@ template <typename T, int WIDTH> class NetworkModule : public Module {
         return grid && network_.supports_grid_input(*grid);
     }
 
-    torch::Tensor inference_with_encoding(const Module &encoding, const torch::Tensor &positions) override {
+    /// a_backward_pass_follows: this is the forward pass of a training step (the batch is then put in cell order from the
+    /// size on from which backward_with_encoding would order it, which can take the order over).
+    torch::Tensor inference_with_encoding(const Module &encoding, const torch::Tensor &positions, bool a_backward_pass_follows = false) override {
         this->enter();
         const tnn_grid_desc *grid = encoding.grid_descriptor();
         if (!grid || !network_.supports_grid_input(*grid))
@@ -336,7 +338,7 @@ template <typename T, int WIDTH> class NetworkModule : public Module {
         if (batch_size == 0) return torch::empty({0, out_w}, torch::TensorOptions().dtype(torch_type<T>::dtype).device(device()));
         torch::Tensor output = torch::empty({(int64_t)batch_size, out_w}, torch::TensorOptions().dtype(torch_type<T>::dtype).device(device()));
         DeviceMatricesView<T> output_network(1, batch_size, network_.get_output_width(), 0, 0, 0, 0, reinterpret_cast<T *>(output.data_ptr()));
-        network_.inference_with_grid(*grid, encoding.grid_table(), positions.data_ptr<float>(), batch_size, output_network);
+        network_.inference_with_grid(*grid, encoding.grid_table(), positions.data_ptr<float>(), batch_size, output_network, a_backward_pass_follows);
         this->finish();
         return output;
     }
@@ -429,7 +431,8 @@ template <typename T, int WIDTH> class NetworkModule : public Module {
     }
 
     std::tuple<torch::Tensor, torch::Tensor> backward_with_encoding(const Module &encoding, const torch::Tensor &positions,
-                                                                    const torch::Tensor &grad_output, bool pack_transpose_gradient) override {
+                                                                    const torch::Tensor &grad_output, bool pack_transpose_gradient,
+                                                                    bool positions_unchanged_since_forward = false) override {
         this->enter();
         const tnn_grid_desc *grid = encoding.grid_descriptor();
         if (!grid || !network_.supports_grid_training(*grid))
@@ -444,7 +447,7 @@ template <typename T, int WIDTH> class NetworkModule : public Module {
         // the scatter overwrites its whole destination: it is the tensor that is handed back
         torch::Tensor table_grad = torch::empty({(int64_t)tnn_grid_n_params(grid), 1}, torch::TensorOptions().dtype(torch::kFloat32).device(device()));
         network_.backward_with_grid(*grid, encoding.grid_table(), positions.data_ptr<float>(), dL_doutput, net_gradients_.GetViews(),
-                                    table_grad.data_ptr<float>());
+                                    table_grad.data_ptr<float>(), positions_unchanged_since_forward);
         return {GradientsTensor(pack_transpose_gradient), table_grad};
     }
 

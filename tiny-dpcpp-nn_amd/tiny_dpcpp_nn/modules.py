@@ -130,7 +130,8 @@ class _EncodedNetworkCall(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, owner, positions, net_params, table):
-        y = owner.network.tnn_module.inference_with_encoding(owner.encoding.tnn_module, positions)
+        # (the native module puts large batches in cell order and keeps the order for the backward pass)
+        y = owner.network.tnn_module.inference_with_encoding(owner.encoding.tnn_module, positions, True)
         ctx.owner = owner
         ctx.save_for_backward(positions, net_params, table)
         return y.reshape(positions.shape[0], -1)[:, : owner.n_output_dims]
@@ -144,7 +145,9 @@ class _EncodedNetworkCall(torch.autograd.Function):
         if scale != 1.0:
             dy = dy * scale
         with torch.no_grad():
-            dnet, dtable = owner.network.tnn_module.bwd_with_encoding(owner.encoding.tnn_module, positions, dy.contiguous(), True)
+            # positions is a tensor autograd saved: it raises if the tensor was written to since the forward pass, so the cell
+            # order formed there (if it was the native module's last) still is the order of these contents
+            dnet, dtable = owner.network.tnn_module.bwd_with_encoding(owner.encoding.tnn_module, positions, dy.contiguous(), True, True)
             if scale != 1.0:
                 dnet = dnet / scale
                 dtable = dtable / scale

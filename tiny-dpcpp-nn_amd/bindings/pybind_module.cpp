@@ -144,6 +144,8 @@ PYBIND11_MODULE(tiny_dpcpp_nn_pybind_module, m) {
         .def("get_params", &PybindingModule::get_params)
         .def("n_output_dims", &PybindingModule::n_output_dims)
         .def("n_params", &PybindingModule::n_params);
+    m.def("set_initial_weight_seed", [](uint64_t seed) { tnn::set_initial_weight_seed(seed); }, py::arg("seed"),
+          "Networks created from now on draw their initial weights from seeds counted up from this one (default: std::random_device, as the reference)");
     m.def("create_network", &create_network_factory, py::arg("input_width"), py::arg("output_width"), py::arg("n_hidden_layers"),
           py::arg("activation"), py::arg("output_activation"), py::arg("width"), py::arg("dtype"), py::arg("use_bias"));
     m.def("create_encoding", &create_encoding_module, py::arg("name"), py::arg("config"), py::arg("padded_output_width") = py::none());

@@ -5,10 +5,37 @@
 // operand-order ("prepared") copies the HIP kernels read, rebuilt whenever the packed weights change.
 #pragma once
 
+#include <atomic>
+#include <cstdint>
 #include <random>
 #include <string>
 
 #include "DeviceMatrix.h"
+
+namespace tnn {
+/// Where the seeds of the initial weights come from: std::random_device, as the reference's (Network.h:262-263 there), until
+/// set_initial_weight_seed() is called; from then on every network takes the next value of a counter that starts at the given
+/// seed, so that a program (a test, a run that is to be repeated) gets the same networks every time.
+struct InitialWeightSeed {
+    static std::atomic<bool> &fixed() {
+        static std::atomic<bool> f{false};
+        return f;
+    }
+    static std::atomic<uint64_t> &counter() {
+        static std::atomic<uint64_t> c{0};
+        return c;
+    }
+    static uint64_t next() {
+        if (fixed().load()) return counter().fetch_add(1);
+        std::random_device entropy;
+        return ((uint64_t)entropy() << 32) | (uint64_t)entropy();
+    }
+};
+inline void set_initial_weight_seed(const uint64_t seed) {
+    InitialWeightSeed::counter().store(seed);
+    InitialWeightSeed::fixed().store(true);
+}
+} // namespace tnn
 
 template <typename T> class NetworkBase {
   public:
@@ -176,7 +203,8 @@ template <typename T> class Network : public NetworkBase<T> {
 
     /// The initial packed weights, drawn on the device. xavier_normal (the reference's name for it) is uniform in
     /// +-sqrt(6 / (fan_in + fan_out)), where the first and the last matrix both count the caller's input width rounded up to
-    /// 16 as one of the two fans (Network.h:278-286 there). The seed comes from std::random_device, as the reference's does.
+    /// 16 as one of the two fans (Network.h:278-286 there). The seed comes from std::random_device, as the reference's does, unless
+    /// tnn::set_initial_weight_seed() fixed it.
     void draw_initial_weights(const WeightInitMode mode) {
         const int dtype = tnn::dtype_of<T>::value;
         switch (mode) {
@@ -187,8 +215,7 @@ template <typename T> class Network : public NetworkBase<T> {
         case WeightInitMode::xavier_normal: break;
         default: throw std::invalid_argument("Invalid weights initialization mode.");
         }
-        std::random_device entropy;
-        const uint64_t seed = ((uint64_t)entropy() << 32) | (uint64_t)entropy();
+        const uint64_t seed = tnn::InitialWeightSeed::next();
         const uint32_t n_mats = m_weights_matrices.GetNumberOfMatrices();
         const int edge_fan = (int)Shape::round_up((int)shape_.raw_in, 16, "Input");
         uint64_t drawn = 0;

@@ -149,7 +149,9 @@ template <typename T> class GridEncodingTemplated : public GridEncoding<T> {
         if (this->m_max_level < (float)m_desc.n_levels) throw std::invalid_argument("GridEncoding: max_level below the level count is not supported.");
     }
 
-    static constexpr size_t kCellOrderMinBatch = size_t(1) << 19; // below this the ordering costs what it saves
+    // below this the ordering costs what it saves (2^18 points: 25 us + 42 us against 76 us in 2-D, 25 + 174 against 224 in 3-D
+    // with a table of 2^22 entries per level; 2^17: 22 + 28 against 40 and 22 + 97 against 115)
+    static constexpr size_t kCellOrderMinBatch = size_t(1) << 18;
     static constexpr size_t kCellOrderMinBackwardBatch = size_t(1) << 17;
 
     tnn_grid_desc m_desc;

@@ -69,7 +69,11 @@ def main():
     ap.add_argument("--batch_size", type=int, default=2 ** 16)
     ap.add_argument("--log2_hashmap_size", type=int, default=15)
     ap.add_argument("--ppm", default=None, help="write the learned 512 x 512 image here")
+    ap.add_argument("--seed", type=int, default=None, help="the same batches and the same initial weights in every run")
     args = ap.parse_args()
+    if args.seed is not None:
+        torch.manual_seed(args.seed)
+        tnn.manual_seed(args.seed)
 
     device = "cuda"
     target = PictureTarget(args.image, device) if args.image else target_image

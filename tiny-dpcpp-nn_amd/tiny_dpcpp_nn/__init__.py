@@ -1,10 +1,11 @@
 """MI355X-native drop-in for the `tiny_dpcpp_nn` Python package of intel/tiny-dpcpp-nn.
 
-Public names are those of the reference (dpcpp_bindings/tiny_dpcpp_nn/__init__.py:1-8). They are resolved on first
+Public names are those of the reference (dpcpp_bindings/tiny_dpcpp_nn/__init__.py:1-8), plus `manual_seed` (reproducible initial
+weights; the reference seeds every network from std::random_device). They are resolved on first
 use, so that `tiny_dpcpp_nn._lib` (the ctypes binding of the C ABI) can be imported without PyTorch.
 """
 
-__all__ = ["free_temporary_memory", "NetworkWithInputEncoding", "Network", "Encoding"]
+__all__ = ["free_temporary_memory", "NetworkWithInputEncoding", "Network", "Encoding", "manual_seed"]
 
 
 def __getattr__(name):

@@ -21,7 +21,7 @@ is not built. There is no PyTorch fallback.
 import torch
 import torch.nn.functional as F
 
-from .tiny_dpcpp_nn_pybind_module import Activation, create_encoding, create_network
+from .tiny_dpcpp_nn_pybind_module import Activation, create_encoding, create_network, set_initial_weight_seed
 
 MIN_BATCH_SIZE = 8  # the kernels take batches that are multiples of 8 rows
 DEFAULT_DEVICE = "cuda"
@@ -29,6 +29,13 @@ DEFAULT_DEVICE = "cuda"
 _ACTIVATIONS = {"relu": Activation.ReLU, "tanh": Activation.Tanh, "sigmoid": Activation.Sigmoid, "linear": Activation.Linear,
                 "none": Activation.Linear}
 _NETWORK_DTYPES = (torch.float16, torch.bfloat16)
+
+
+def manual_seed(seed):
+    """Networks created from now on get reproducible initial weights: seeds counted up from `seed`. Without this call every
+    network is seeded from std::random_device, as in the reference (include/network/Network.h:262-263 there), and two runs of a
+    program train different networks. No counterpart in the reference."""
+    set_initial_weight_seed(int(seed) & (2 ** 64 - 1))
 
 
 def free_temporary_memory():
